@@ -70,10 +70,21 @@ class TorchOps:
     def place_tokens(self, ids, dest, source, tokens, count):
         ids[dest[:count].long()] = tokens[source[:count].long()]
 
-    def embed(self, token_ids, table):
-        return table[token_ids.long()].float()
+    def embed(self, token_ids, table, scale=1.0):
+        out = table[token_ids.long()].float()
+        return out * scale if scale != 1.0 else out
+
+    @staticmethod
+    def _one_delta(delta):
+        from velox_amd.parts.base import SumOf
+
+        if isinstance(delta, SumOf):
+            first = delta.first.float().sum(0) if delta.first.dim() == 3 else delta.first.float()
+            return first + delta.second.float()
+        return delta
 
     def add_rmsnorm(self, residual, delta, weight, eps, out_dtype):
+        delta = self._one_delta(delta)
         if delta is not None and delta.dim() == 3:
             delta = delta.float().sum(0)
         if delta is not None:
@@ -82,6 +93,7 @@ class TorchOps:
         return (residual * torch.rsqrt(var + eps) * weight.float()).to(out_dtype)
 
     def add_rmsnorm_rows(self, residual, delta, rows, weight, eps, out_dtype):
+        delta = self._one_delta(delta)
         if delta is not None and delta.dim() == 3:
             delta = delta.float().sum(0)
         x = residual[rows.long()]
@@ -132,6 +144,91 @@ class TorchOps:
             offsets = (slot_mapping.long() % block_size)
             k_cache[pages, :, offsets, :] = k.to(k_cache.dtype)
             v_cache[pages, :, :, offsets] = v.to(v_cache.dtype)
+
+    # -- attention over a cached latent ---------------------------------------------------
+    @staticmethod
+    def _rotate(x, cos, sin, interleaved):
+        """``x`` float32 [T, ..., n]; rotates its first 2 * table width channels."""
+        half = cos.shape[-1]
+        while cos.dim() < x.dim():
+            cos, sin = cos.unsqueeze(1), sin.unsqueeze(1)
+        out = x.clone()
+        if interleaved:
+            u, v = x[..., 0:2 * half:2], x[..., 1:2 * half:2]
+            out[..., 0:2 * half:2] = u * cos - v * sin
+            out[..., 1:2 * half:2] = v * cos + u * sin
+        else:
+            u, v = x[..., :half], x[..., half:2 * half]
+            out[..., :half] = u * cos - v * sin
+            out[..., half:2 * half] = v * cos + u * sin
+        return out
+
+    def latent_rotate_write(self, projected, num_heads, dim, rot_dim, kv_rank, cached_dim, down_offset, positions, cos, sin, interleaved,
+                            norm_weight, eps, slot_mapping, k_cache, v_cache, block_size):
+        t = projected.shape[0]
+        wide = projected.float()
+        c = s = None
+        if cos is not None:
+            c, s = cos[positions.long()], sin[positions.long()]
+        queries = torch.zeros((t, num_heads, cached_dim), dtype=projected.dtype, device=projected.device)
+        turned = wide[:, : num_heads * (dim + rot_dim)].view(t, num_heads, dim + rot_dim)[..., dim:]
+        if c is not None:
+            turned = self._rotate(turned, c, s, interleaved)
+        queries[..., kv_rank:kv_rank + rot_dim] = turned.to(projected.dtype)
+        if down_offset >= 0:
+            latent = wide[:, down_offset:down_offset + kv_rank]
+            latent = latent / torch.sqrt((latent * latent).mean(-1, keepdim=True) + eps) * norm_weight.float()
+            shared = wide[:, down_offset + kv_rank:down_offset + kv_rank + rot_dim]
+            if c is not None:
+                shared = self._rotate(shared, c, s, interleaved)
+            row = torch.zeros((t, cached_dim), dtype=k_cache.dtype, device=projected.device)
+            row[:, :kv_rank] = latent.to(k_cache.dtype)
+            row[:, kv_rank:kv_rank + rot_dim] = shared.to(k_cache.dtype)
+            pages = slot_mapping.long() // block_size
+            offsets = slot_mapping.long() % block_size
+            k_cache[pages, 0, offsets, :] = row
+            v_cache[pages, 0, :, offsets] = row
+        return queries.view(t, num_heads * cached_dim)
+
+    def head_linear(self, x, x_head_stride, x_offset, maps, out, out_head_stride, out_offset, gate=None, gate_offset=0):
+        groups, n, k = maps.shape
+        t = x.shape[0]
+        for g in range(groups):
+            a = x[:, g * x_head_stride + x_offset:g * x_head_stride + x_offset + k].float()
+            y = a @ maps[g].float().T
+            if gate is not None:
+                y = y * torch.sigmoid(gate[:, gate_offset + g * n:gate_offset + (g + 1) * n].float())
+            out[:, g * out_head_stride + out_offset:g * out_head_stride + out_offset + n] = y.to(out.dtype)
+        return out
+
+    # -- routed experts -------------------------------------------------------------------
+    def route_top(self, logits, top, score="sigmoid", renormalize=False):
+        scores = torch.sigmoid(logits.float()) if score == "sigmoid" else torch.softmax(logits.float(), dim=-1)
+        weight, choice = scores.topk(top, dim=-1)
+        if renormalize:
+            weight = weight / weight.sum(-1, keepdim=True)
+        return choice.to(torch.int32), weight
+
+    def routed_experts(self, x, choice, weight, gate_up_weight, down_weight, num_experts, scale_input, shared, out_dtype, workspace=None):
+        t, h = x.shape
+        f = gate_up_weight.shape[0] // (2 * num_experts)
+        gate_up = gate_up_weight.view(num_experts, 2 * f, h).float()
+        down = down_weight.view(num_experts, h, f).float()
+        out = torch.zeros((t, h), dtype=torch.float32, device=x.device)
+        for k in range(choice.shape[1]):  # a token's results are added in the order of its choices
+            for e in range(num_experts):
+                rows = (choice[:, k] == e).nonzero().flatten()
+                if not rows.numel():
+                    continue
+                w = weight[rows, k:k + 1]
+                a = (x[rows].float() * w).to(x.dtype).float() if scale_input else x[rows].float()
+                both = a @ gate_up[e].T
+                act = (both[:, :f] * torch.sigmoid(both[:, :f]) * both[:, f:]).to(x.dtype).float()
+                y = act @ down[e].T
+                out[rows] += y if scale_input else y * w
+        if shared is not None:
+            out = out + shared.float()
+        return out.to(out_dtype)
 
     # -- attention over the paged cache -------------------------------------------------
     def paged_attention(self, qkv, num_heads, num_kv_heads, head_dim, k_cache, v_cache, block_size, block_tables, cu_q, kv_lens, max_q_len, max_kv_len, scale, window, all_decode, workspace, splits=None, decode_prefix=0, portions_max_kv_len=None):

@@ -35,11 +35,13 @@ def architecture_name(raw: Dict[str, Any]) -> str:
     names = raw.get("architectures")
     if names and isinstance(names, (list, tuple)) and isinstance(names[0], str):
         return names[0]
+    if isinstance(raw.get("architecture"), str):  # (some configurations name their one class under this key)
+        return raw["architecture"]
     _load_builtin()
     model_type = raw.get("model_type")
     if isinstance(model_type, str) and model_type in _ARCHITECTURE_OF_MODEL_TYPE:
         return _ARCHITECTURE_OF_MODEL_TYPE[model_type]
-    raise ConfigError('config.json must name its model class in "architectures" (or a known "model_type")')
+    raise ConfigError('config.json must name its model class in "architectures" or "architecture" (or a known "model_type")')
 
 
 def known_architectures():

@@ -51,6 +51,8 @@ class AttentionMixer(Mixer):
             raise ValueError(f"head_dim={head_dim}: the attention kernels take multiples of 16 from 16 to 256")
         if window is not None and window < 1:
             raise ValueError(f"window={window} must be at least 1")
+        if getattr(position, "layout", "halves") != "halves":
+            raise ValueError("this mixer's rotation kernels pair channels (i, i + d/2); an interleaved rotation belongs to another mixer")
         self.hidden_size = int(hidden_size)
         self.num_heads = int(num_heads)
         self.num_kv_heads = int(num_kv_heads)

@@ -192,6 +192,16 @@ class ResidualSink:
 
 
 @dataclass
+class SumOf:
+    """What a block whose sub-layers run side by side hands to the next norm: ``first + second`` is the block's output.
+    ``first`` is ``[T, H]`` or float32 partial sums ``[S, T, H]``, ``second`` is ``[T, H]``; the norm's kernel adds them to
+    each other in float32 and the sum to the residual, so the residual gets ``x + (a + b)`` with one rounding each."""
+
+    first: torch.Tensor
+    second: torch.Tensor
+
+
+@dataclass
 class DeferredNorm:
     """Normalised activations that have not been computed as such: ``x`` holds ``residual * weight`` in the run dtype and
     ``sums`` what is needed for each row's ``rsqrt(mean(residual^2) + eps)``; the products that read them
@@ -243,8 +253,8 @@ class Norm(Part):
     def forward(self, residual: torch.Tensor, delta: Optional[torch.Tensor], ctx, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
         """``residual`` [T, H] float32.
 
-        ``delta`` is [T, H] or float32 partial sums [S, T, H], which are added first to last, or a ``DeferredNorm`` made
-        for this very norm (then the residual is up to date and the ``DeferredNorm`` itself is what comes back).
+        ``delta`` is [T, H] or float32 partial sums [S, T, H], which are added first to last, or a ``SumOf`` two such
+        terms, or a ``DeferredNorm`` made for this very norm (then the residual is up to date and the ``DeferredNorm`` itself is what comes back).
         With ``rows`` None: ``residual += delta`` in place (delta may be None) and the
         normalised residual comes back in the run dtype, [T, H].  With ``rows`` (int32
         [R]): nothing is changed and ``normalise(residual[rows] + delta[rows])`` comes back.

@@ -1,9 +1,12 @@
-"""Arrangement of one mixer and one feed-forward with their norms.
+"""Arrangements of one mixer and one feed-forward with their norms.
 
 ``PreNormBlock`` is the reference's ``DecoderLayer.forward`` (``src/decoder_layer.py:41-54``):
 ``h = h + mixer(norm1(h)); h = h + ff(norm2(h))``.  The residual ``h`` lives in a float32
 tensor; what a sub-layer produced is carried as ``pending`` and added inside the next
 norm's kernel, so each block hands its feed-forward output on to whoever normalises next.
+
+``ParallelBlock`` (not in the reference): ``n = norm(h); h = h + (mixer(n) + ff(n))``, one norm that both
+sub-layers read.  It hands both outputs on as a ``SumOf``, which the next norm's kernel adds up in float32.
 """
 from __future__ import annotations
 
@@ -11,7 +14,7 @@ from typing import Optional, Tuple
 
 import torch
 
-from .base import Block, FeedForward, Mixer, Norm, Part, ResidualSink, register_arrangement
+from .base import Block, FeedForward, Mixer, Norm, Part, ResidualSink, SumOf, register_arrangement
 
 
 class PreNormBlock(Block):
@@ -47,3 +50,33 @@ class PreNormBlock(Block):
 
 
 register_arrangement("pre_norm", PreNormBlock)
+
+
+class ParallelBlock(Block):
+    def __init__(self, prefix: str, mixer: Mixer, feed_forward: FeedForward, mixer_norm: Norm, ff_norm: Optional[Norm] = None) -> None:
+        """``ff_norm`` is not used and owns no tensors here: there is one norm."""
+        super().__init__(prefix)
+        self.mixer = mixer
+        self.feed_forward = feed_forward
+        self.norm = mixer_norm
+
+    def children(self) -> Tuple[Part, ...]:
+        return (self.norm, self.mixer, self.feed_forward)
+
+    def input_norm(self) -> Optional[Norm]:
+        return self.norm
+
+    def forward(self, residual: torch.Tensor, pending, ctx, cache, owns_cache: bool, next_norm: Optional[Norm] = None):
+        normed = ctx.ops.materialize(self.norm.forward(residual, pending, ctx))
+        mixed = self.mixer.forward(normed, ctx, cache, owns_cache)
+        other = self.feed_forward.forward(normed, ctx)
+        if other is None:
+            return mixed
+        if other.dim() == 3:
+            mixed, other = other, mixed  # (the term that may be partial sums goes first)
+        if other.dim() == 3:
+            other = other.sum(0)
+        return SumOf(mixed, other)
+
+
+register_arrangement("parallel", ParallelBlock)

@@ -1,14 +1,21 @@
-"""Dense gated feed-forward.
+"""Feed-forwards: the dense gated one, routed experts, and none at all.
 
 Reference ``src/mlp.py:9-15``: one fused product with rows ``[Wgate; Wup]`` (no bias),
 ``act(gate) * up``, down product (no bias); ``silu(x) = x * sigmoid(x)``.  The
 activation and the product ``act(gate) * up`` are computed in float32 with one
 rounding at the store; for decode-sized batches they are the epilogue of the
 gate/up product itself, which then never writes its ``[T, 2I]`` result.
+
+``RoutedExperts`` (no counterpart in the reference): ``E`` small gated units of which every token uses ``top``,
+chosen by a router whose logits are float32.  The score function, whether the chosen scores are renormalised and
+whether a score scales the expert's input or its output are options of the part.  Nothing is decided on the host:
+a plan kernel sorts the (token, choice) pairs by expert on the device, two grouped products run every expert on
+its own rows, and a last kernel adds each token's results in the order of its choices, so the step can be captured
+and a token's result does not depend on which other tokens share its experts.
 """
 from __future__ import annotations
 
-from typing import Dict, Optional
+from typing import Dict, Optional, Tuple
 
 import torch
 
@@ -16,8 +23,11 @@ from .base import FeedForward, Param, fused_rows, register_part, single
 
 
 class GatedMLP(FeedForward):
-    def __init__(self, prefix: str, hidden_size: int, intermediate_size: int, activation: str = "silu") -> None:
+    def __init__(self, prefix: str, hidden_size: int, intermediate_size: int, activation: str = "silu",
+                 names: Tuple[str, str, str] = ("gate_proj.weight", "up_proj.weight", "down_proj.weight")) -> None:
+        """``names``: the gate, up and down tensors below the prefix."""
         super().__init__(prefix)
+        self.names = tuple(names)
         if activation != "silu":
             raise ValueError(f"activation {activation!r} is not implemented (only 'silu')")
         self.hidden_size = int(hidden_size)
@@ -28,8 +38,8 @@ class GatedMLP(FeedForward):
     def params(self) -> Dict[str, Param]:
         h, i = self.hidden_size, self.intermediate_size
         return {
-            "gate_up_weight": fused_rows(("gate_proj.weight", "up_proj.weight"), ((i, h), (i, h))),
-            "down_weight": single("down_proj.weight", (h, i)),
+            "gate_up_weight": fused_rows(self.names[:2], ((i, h), (i, h))),
+            "down_weight": single(self.names[2], (h, i)),
         }
 
     def prepare_kernels(self, ops) -> None:
@@ -46,3 +56,86 @@ class GatedMLP(FeedForward):
 
 
 register_part("feed_forward", "gated_mlp", GatedMLP)
+
+
+class NoFeedForward(FeedForward):
+    """A layer without a feed-forward: ``forward`` gives None and the block adds nothing."""
+
+    def __init__(self, prefix: str = "") -> None:
+        super().__init__(prefix)
+
+    def forward(self, x, ctx, sink=None):
+        return None
+
+
+register_part("feed_forward", "none", NoFeedForward)
+
+
+class RoutedExperts(FeedForward):
+    """``y = sum_k unit_{e_k}(s_k x)`` (``scale_input``) or ``sum_k s_k unit_{e_k}(x)``, plus ``shared(x)`` when there is
+    a shared unit; ``unit(x) = W_down (silu(W_gate x) * (W_up x))``; ``e_1 .. e_top`` are the experts with the largest
+    scores ``s = score(W_router x)`` (``sigmoid``, or ``softmax`` over all experts), kept as they are or divided by their
+    sum (``renormalize``).  The router's logits and the scores are float32.
+
+    Tensors: the experts' gate and up matrices are held as one ``[E * 2 F, H]`` tensor (expert after expert, each gate
+    rows then up rows), the down matrices as ``[E * H, F]``; ``expert_names(e)`` gives the three names of expert ``e``
+    below the prefix."""
+
+    def __init__(self, prefix: str, hidden_size: int, intermediate_size: int, num_experts: int, top: int, score: str = "sigmoid",
+                 renormalize: bool = False, scale_input: bool = True, shared_intermediate_size: Optional[int] = None,
+                 expert_names: Tuple[str, str, str] = ("experts.{e}.gate.weight", "experts.{e}.up.weight", "experts.{e}.down.weight"),
+                 router_name: str = "router.weight", shared_prefix: str = "shared.",
+                 shared_names: Tuple[str, str, str] = ("gate_proj.weight", "up_proj.weight", "down_proj.weight")) -> None:
+        super().__init__(prefix)
+        if score not in ("sigmoid", "softmax"):
+            raise ValueError(f"score {score!r} is not implemented ('sigmoid' or 'softmax')")
+        if not 1 <= int(top) <= int(num_experts):
+            raise ValueError(f"top={top} must lie between 1 and the number of experts ({num_experts})")
+        self.hidden_size = int(hidden_size)
+        self.intermediate_size = int(intermediate_size)
+        self.num_experts = int(num_experts)
+        self.top = int(top)
+        self.score = score
+        self.renormalize = bool(renormalize)
+        self.scale_input = bool(scale_input)
+        self.expert_names = tuple(expert_names)
+        self.router_name = router_name
+        self.shared = None
+        if shared_intermediate_size:
+            self.shared = GatedMLP(prefix + shared_prefix, hidden_size, int(shared_intermediate_size), names=shared_names)
+        self.router_weight: Optional[torch.Tensor] = None
+        self.gate_up_weight: Optional[torch.Tensor] = None
+        self.down_weight: Optional[torch.Tensor] = None
+
+    def params(self) -> Dict[str, Param]:
+        h, f, e = self.hidden_size, self.intermediate_size, self.num_experts
+        gate, up, down = self.expert_names
+        gate_up_names = tuple(name.format(e=i) for i in range(e) for name in (gate, up))
+        return {
+            "router_weight": single(self.router_name, (e, h)),
+            "gate_up_weight": fused_rows(gate_up_names, ((f, h),) * (2 * e)),
+            "down_weight": fused_rows(tuple(down.format(e=i) for i in range(e)), ((h, f),) * e),
+        }
+
+    def children(self):
+        return (self.shared,) if self.shared is not None else ()
+
+    def workspace_needs(self, ops, limits):
+        sizes = getattr(ops, "routed_plan_elems", None)
+        if sizes is None:
+            return {}
+        return {"routed_plan": sizes(limits.max_num_tokens, self.top, self.num_experts)}
+
+    def forward(self, x, ctx, sink=None):
+        ops = ctx.ops
+        x = ops.materialize(x)
+        logits = ops.linear(x, self.router_weight, None, torch.float32)
+        choice, weight = ops.route_top(logits, self.top, self.score, self.renormalize)
+        shared = self.shared.forward(x, ctx) if self.shared is not None else None
+        if shared is not None and shared.dim() == 3:
+            shared = shared.sum(0)  # (partial sums of a split product; the experts' results are added to one tensor)
+        return ops.routed_experts(x, choice, weight, self.gate_up_weight, self.down_weight, self.num_experts, self.scale_input, shared,
+                                  ctx.dtype, ctx.workspace)
+
+
+register_part("feed_forward", "routed_experts", RoutedExperts)

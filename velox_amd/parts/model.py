@@ -81,20 +81,24 @@ class ModelSpec:
 
 
 class TableEmbedding(Embedding):
-    """``h[t] = E[ids[t]]``, no scaling (reference ``src/transformer.py:27,44``)."""
+    """``h[t] = E[ids[t]] * scale``; the reference has no scaling (``src/transformer.py:27,44``), which is ``scale`` = 1.
+    The product is taken in float32, inside the kernel that looks the rows up."""
 
-    def __init__(self, name: str, vocab_size: int, hidden_size: int) -> None:
+    def __init__(self, name: str, vocab_size: int, hidden_size: int, scale: float = 1.0) -> None:
         super().__init__("")
         self.name = name
         self.vocab_size = vocab_size
         self.hidden_size = hidden_size
+        self.scale = float(scale)
         self.table: Optional[torch.Tensor] = None
 
     def params(self) -> Dict[str, Param]:
         return {"table": single(self.name, (self.vocab_size, self.hidden_size), product=False)}
 
     def forward(self, token_ids: torch.Tensor, ctx) -> torch.Tensor:
-        return ctx.ops.embed(token_ids, self.table)
+        if self.scale == 1.0:
+            return ctx.ops.embed(token_ids, self.table)
+        return ctx.ops.embed(token_ids, self.table, scale=self.scale)
 
 
 class LinearHead(OutputHead):

@@ -16,14 +16,17 @@ from .base import DeferredNorm, Norm, Param, register_part, single
 
 
 class RMSNorm(Norm):
-    def __init__(self, prefix: str, hidden_size: int, eps: float) -> None:
+    def __init__(self, prefix: str, hidden_size: int, eps: float, weight_name: str = "weight") -> None:
+        """``weight_name``: the tensor's name below the prefix (an architecture whose checkpoint names the norm's
+        weight by the prefix alone passes "")."""
         super().__init__(prefix)
         self.hidden_size = int(hidden_size)
         self.eps = float(eps)
+        self.weight_name = weight_name
         self.weight: Optional[torch.Tensor] = None
 
     def params(self) -> Dict[str, Param]:
-        return {"weight": single("weight", (self.hidden_size,), role="vector", init="one_plus_normal")}
+        return {"weight": single(self.weight_name, (self.hidden_size,), role="vector", init="one_plus_normal")}
 
     def deferred_form(self):
         return self.weight, self.eps

@@ -7,10 +7,20 @@ run dtype (``src/rope.py:58-63``).  The rotation itself (halves paired ``(i, i +
 ``src/rope_inplace.py:25-47``) is fused into the attention mixer's cache-write kernel.
 The tables are built on the host so that every run, on any device, rotates by
 bit-identical angles.
+
+Two options beyond the reference's: ``layout`` says which channels are a pair (``halves``:
+``(i, i + d/2)``; ``interleaved``: ``(2i, 2i + 1)``; the mixer's rotation kernel reads it), and
+``stretch = (factor, original, fast, slow)`` stretches the slow frequencies for contexts beyond the
+``original`` length (YaRN): with ``dim(t) = d ln(original / (2 pi t)) / (2 ln theta)``,
+``lo = max(floor(dim(fast)), 0)``, ``hi = min(ceil(dim(slow)), d - 1)`` and
+``r_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1)`` the frequency becomes
+``f_i / factor * r_i + f_i (1 - r_i)``, and cos and sin are both multiplied by
+``0.1 ln(factor) + 1``, which the tables hold already.
 """
 from __future__ import annotations
 
-from typing import Optional, Tuple
+import math
+from typing import Optional, Sequence, Tuple
 
 import torch
 
@@ -18,10 +28,17 @@ from .base import PositionEncoding, register_part
 
 
 class RotaryEncoding(PositionEncoding):
-    def __init__(self, rotary_dim: int, theta: float, max_position: int, scaling_factor: float = 1.0) -> None:
+    def __init__(self, rotary_dim: int, theta: float, max_position: int, scaling_factor: float = 1.0, layout: str = "halves",
+                 stretch: Optional[Sequence[float]] = None) -> None:
         super().__init__("")
         if rotary_dim % 2 != 0:
             raise ValueError(f"rotary_dim must be even, got {rotary_dim}")
+        if layout not in ("halves", "interleaved"):
+            raise ValueError(f"layout must be 'halves' or 'interleaved', got {layout!r}")
+        if stretch is not None and (len(stretch) != 4 or not stretch[0] > 0 or not stretch[1] > 0 or not stretch[2] > 0 or not stretch[3] > 0):
+            raise ValueError(f"stretch must be four positive numbers (factor, original, fast, slow), got {stretch!r}")
+        self.layout = layout
+        self.stretch = tuple(float(v) for v in stretch) if stretch is not None else None
         self.rotary_dim = int(rotary_dim)
         self.theta = float(theta)
         self.max_position = int(max_position)
@@ -29,15 +46,35 @@ class RotaryEncoding(PositionEncoding):
         self.cos: Optional[torch.Tensor] = None
         self.sin: Optional[torch.Tensor] = None
 
+    def frequencies(self) -> Tuple[torch.Tensor, float]:
+        """float32 ``[rotary_dim / 2]`` and the factor that cos and sin are multiplied with."""
+        if self.stretch is None:
+            exponent = torch.arange(0, self.rotary_dim, 2, dtype=torch.float32) / self.rotary_dim
+            return 1.0 / (self.theta ** exponent), 1.0
+        factor, original, fast, slow = self.stretch
+        d = self.rotary_dim
+        index = torch.arange(d // 2, dtype=torch.float64)
+        plain = self.theta ** (-2.0 * index / d)
+
+        def dim_of(turns: float) -> float:
+            return d * math.log(original / (2.0 * math.pi * turns)) / (2.0 * math.log(self.theta))
+
+        lo = max(math.floor(dim_of(fast)), 0)
+        hi = min(math.ceil(dim_of(slow)), d - 1)
+        ramp = ((index - lo) / max(hi - lo, 0.001)).clamp(0.0, 1.0)
+        return (plain / factor * ramp + plain * (1.0 - ramp)).float(), 0.1 * math.log(factor) + 1.0
+
     def finalize(self, device, dtype) -> None:
-        exponent = torch.arange(0, self.rotary_dim, 2, dtype=torch.float32) / self.rotary_dim
-        inv_freq = 1.0 / (self.theta ** exponent)
+        inv_freq, magnitude = self.frequencies()
         positions = torch.arange(self.max_position, dtype=torch.float32)
         if self.scaling_factor != 1.0:
             positions = positions / self.scaling_factor
         angles = torch.outer(positions, inv_freq)
-        self.cos = angles.cos().contiguous().to(device)
-        self.sin = angles.sin().contiguous().to(device)
+        cos, sin = angles.cos(), angles.sin()
+        if magnitude != 1.0:
+            cos, sin = cos * magnitude, sin * magnitude
+        self.cos = cos.contiguous().to(device)
+        self.sin = sin.contiguous().to(device)
 
     def rotary_tables(self) -> Optional[Tuple[torch.Tensor, torch.Tensor]]:
         return self.cos, self.sin
