@@ -72,4 +72,25 @@ template <int N> __device__ __forceinline__ void wait_for_loads() {
   asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
 }
 
+// Four consecutive elements of a row, widened to float32: one 8- or 16-byte access when `vec_ok` (the row starts on such a
+// boundary and k is a multiple of 4) and all four lie below k_limit, else element by element with zeros beyond k_limit.
+template <typename T>
+__device__ __forceinline__ void load4(const T* __restrict__ base, size_t row_offset, int k, int k_limit, bool row_ok, bool vec_ok, float (&v)[4]) {
+  if (!row_ok) { v[0] = v[1] = v[2] = v[3] = 0.f; return; }
+  const T* p = base + row_offset + k;
+  if (vec_ok && k + 3 < k_limit) {
+    if constexpr (sizeof(T) == 4) {
+      const float4_t x = *reinterpret_cast<const float4_t*>(p);
+      v[0] = x[0]; v[1] = x[1]; v[2] = x[2]; v[3] = x[3];
+    } else {
+      const short4_t x = *reinterpret_cast<const short4_t*>(p);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v[i] = __uint_as_float(((uint32_t)(uint16_t)x[i]) << 16);
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] = (k + i < k_limit) ? to_f32(p[i]) : 0.f;
+  }
+}
+
 #define VELOX_RETURN_LAUNCH_STATUS() return (int)hipGetLastError()

@@ -4,10 +4,10 @@
 #include "common.h"
 
 // ---------------------------------------------------------------------------------------------
-// embedding: out[t, :] = float(table[ids[t], :]); an id outside the table yields NaN rows.
+// embedding: out[t, :] = float(table[ids[t], :]) * scale; an id outside the table yields NaN rows.
 // ---------------------------------------------------------------------------------------------
 template <typename T>
-__global__ void embed_kernel(const int* __restrict__ ids, const T* __restrict__ table, float* __restrict__ out, int hidden, int vocab) {
+__global__ void embed_kernel(const int* __restrict__ ids, const T* __restrict__ table, float* __restrict__ out, int hidden, int vocab, float scale) {
   const int t = blockIdx.x;
   const int id = ids[t];
   float* dst = out + (size_t)t * hidden;
@@ -16,15 +16,16 @@ __global__ void embed_kernel(const int* __restrict__ ids, const T* __restrict__ 
     return;
   }
   const T* src = table + (size_t)id * hidden;
-  for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = to_f32(src[i]);
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = to_f32(src[i]) * scale;
 }
 
-extern "C" int velox_embed(const int* ids, const void* table, float* out, int tokens, int hidden, int vocab, int table_dtype, hipStream_t stream) {
+extern "C" int velox_embed(const int* ids, const void* table, float* out, int tokens, int hidden, int vocab, int table_dtype, float scale,
+                           hipStream_t stream) {
   if (tokens <= 0) return 0;
   if (table_dtype == VELOX_BF16)
-    embed_kernel<bf16_t><<<tokens, 256, 0, stream>>>(ids, (const bf16_t*)table, out, hidden, vocab);
+    embed_kernel<bf16_t><<<tokens, 256, 0, stream>>>(ids, (const bf16_t*)table, out, hidden, vocab, scale);
   else
-    embed_kernel<float><<<tokens, 256, 0, stream>>>(ids, (const float*)table, out, hidden, vocab);
+    embed_kernel<float><<<tokens, 256, 0, stream>>>(ids, (const float*)table, out, hidden, vocab, scale);
   VELOX_RETURN_LAUNCH_STATUS();
 }
 
@@ -53,10 +54,16 @@ extern "C" int velox_place_tokens(int* ids, const int* dest, const int* source, 
 // ---------------------------------------------------------------------------------------------
 //   delta may be `partials` stacked tensors (partial sums of a split product), `partial_stride` elements apart: they are
 //   added in order, first to last.
+//   With `second` (a [T, H] tensor, bfloat16 if second_bf16 else float32) the delta is a sum of two terms: the partial
+//   sums and `second` are added to each other first and their sum to the residual, r = residual + ((p0 + p1 + ..) + second).
+__device__ __forceinline__ float second_at(const void* second, int second_bf16, size_t index) {
+  return second_bf16 ? to_f32(((const bf16_t*)second)[index]) : ((const float*)second)[index];
+}
+
 template <typename TD, typename TO>
 __global__ void add_rmsnorm_kernel(float* __restrict__ residual, const TD* __restrict__ delta, const int* __restrict__ rows,
                                    const float* __restrict__ weight, TO* __restrict__ out, int hidden, float eps,
-                                   int partials, size_t partial_stride) {
+                                   int partials, size_t partial_stride, const void* __restrict__ second, int second_bf16) {
   __shared__ float scratch[16];
   const int row = blockIdx.x;
   const size_t src_row = rows ? (size_t)rows[row] : (size_t)row;
@@ -66,8 +73,13 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ residual, const TD* __res
   float sumsq = 0.f;
   for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
     float r = res[i];
-    if (del)
+    if (del && second) {
+      float d = 0.f;
+      for (int p = 0; p < partials; ++p) d += to_f32(del[p * partial_stride + i]);
+      r += d + second_at(second, second_bf16, src_row * hidden + i);
+    } else if (del) {
       for (int p = 0; p < partials; ++p) r += to_f32(del[p * partial_stride + i]);
+    }
     if (write_back) res[i] = r;
     sumsq += r * r;
   }
@@ -76,8 +88,15 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ residual, const TD* __res
   TO* dst = out + (size_t)row * hidden;
   for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
     float r = res[i];
-    if (del && !write_back)
-      for (int p = 0; p < partials; ++p) r += to_f32(del[p * partial_stride + i]);
+    if (del && !write_back) {
+      if (second) {
+        float d = 0.f;
+        for (int p = 0; p < partials; ++p) d += to_f32(del[p * partial_stride + i]);
+        r += d + second_at(second, second_bf16, src_row * hidden + i);
+      } else {
+        for (int p = 0; p < partials; ++p) r += to_f32(del[p * partial_stride + i]);
+      }
+    }
     dst[i] = from_f32<TO>(r * inv * weight[i]);
   }
 }
@@ -99,7 +118,7 @@ template <> struct Quad<bf16_t> {
 template <typename TD, typename TO, int CHUNKS>
 __global__ void add_rmsnorm_rows_in_registers_kernel(float* __restrict__ residual, const TD* __restrict__ delta, const int* __restrict__ rows,
                                                      const float* __restrict__ weight, TO* __restrict__ out, int hidden, float eps,
-                                                     int partials, size_t partial_stride) {
+                                                     int partials, size_t partial_stride, const void* __restrict__ second, int second_bf16) {
   __shared__ float scratch[16];
   const int row = blockIdx.x;
   const size_t src_row = rows ? (size_t)rows[row] : (size_t)row;
@@ -114,7 +133,17 @@ __global__ void add_rmsnorm_rows_in_registers_kernel(float* __restrict__ residua
     r[c] = float4_t{0.f, 0.f, 0.f, 0.f};
     if (at < hidden) {
       r[c] = *reinterpret_cast<const float4_t*>(res + at);
-      if (del) {
+      if (del && second) {
+        // two terms: the partial sums and `second` are added to each other first, then to the residual
+        float4_t d = float4_t{0.f, 0.f, 0.f, 0.f};
+        for (int p = 0; p < partials; ++p) {
+          const Quad<TD> q = *reinterpret_cast<const Quad<TD>*>(del + p * partial_stride + at);
+#pragma unroll
+          for (int j = 0; j < 4; ++j) d[j] += q.get(j);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) r[c][j] += d[j] + second_at(second, second_bf16, src_row * hidden + at + j);
+      } else if (del) {
         // four partial sums are asked for together (the last one again where fewer are left) and added in order
         for (int p = 0; p < partials; p += 4) {
           Quad<TD> d[4];
@@ -155,18 +184,19 @@ __global__ void add_rmsnorm_rows_in_registers_kernel(float* __restrict__ residua
 
 extern "C" int velox_add_rmsnorm(float* residual, const void* delta, const int* rows, const float* weight, void* out,
                                  int num_rows, int hidden, float eps, int delta_dtype, int out_dtype, int partials,
-                                 long long partial_stride, hipStream_t stream) {
+                                 long long partial_stride, const void* second, int second_dtype, hipStream_t stream) {
   if (num_rows <= 0) return 0;
-  if (partials < 1 || (partials > 1 && partial_stride % 4 != 0)) return -1;
+  if (partials < 1 || (partials > 1 && partial_stride % 4 != 0) || (second != nullptr && delta == nullptr)) return -1;
+  const int second_bf16 = second_dtype == VELOX_BF16;
   const int threads = hidden >= 2048 ? 512 : 256;
   const bool aligned = (((uintptr_t)residual | (uintptr_t)delta | (uintptr_t)weight | (uintptr_t)out) & 15) == 0;
   const bool in_registers = aligned && hidden % 4 == 0 && hidden <= 4 * threads * 4;
 #define LAUNCH(TD, TO)                                                                                                                  \
   do {                                                                                                                                  \
     if (in_registers)                                                                                                                   \
-      add_rmsnorm_rows_in_registers_kernel<TD, TO, 4><<<num_rows, threads, 0, stream>>>(residual, (const TD*)delta, rows, weight, (TO*)out, hidden, eps, partials, (size_t)partial_stride); \
+      add_rmsnorm_rows_in_registers_kernel<TD, TO, 4><<<num_rows, threads, 0, stream>>>(residual, (const TD*)delta, rows, weight, (TO*)out, hidden, eps, partials, (size_t)partial_stride, second, second_bf16); \
     else                                                                                                                                \
-      add_rmsnorm_kernel<TD, TO><<<num_rows, threads, 0, stream>>>(residual, (const TD*)delta, rows, weight, (TO*)out, hidden, eps, partials, (size_t)partial_stride); \
+      add_rmsnorm_kernel<TD, TO><<<num_rows, threads, 0, stream>>>(residual, (const TD*)delta, rows, weight, (TO*)out, hidden, eps, partials, (size_t)partial_stride, second, second_bf16); \
   } while (0)
   if (delta_dtype == VELOX_BF16 && out_dtype == VELOX_BF16) LAUNCH(bf16_t, bf16_t);
   else if (delta_dtype == VELOX_F32 && out_dtype == VELOX_F32) LAUNCH(float, float);

@@ -17,25 +17,6 @@
 #define GEMM_PAD 4
 #define GEMM_FOLD 128  // terms per inner sum (a multiple of GEMM_BK)
 
-template <typename T>
-__device__ __forceinline__ void load4(const T* __restrict__ base, size_t row_offset, int k, int k_limit, bool row_ok, bool vec_ok, float (&v)[4]) {
-  if (!row_ok) { v[0] = v[1] = v[2] = v[3] = 0.f; return; }
-  const T* p = base + row_offset + k;
-  if (vec_ok && k + 3 < k_limit) {
-    if constexpr (sizeof(T) == 4) {
-      const float4_t x = *reinterpret_cast<const float4_t*>(p);
-      v[0] = x[0]; v[1] = x[1]; v[2] = x[2]; v[3] = x[3];
-    } else {
-      const short4_t x = *reinterpret_cast<const short4_t*>(p);
-#pragma unroll
-      for (int i = 0; i < 4; ++i) v[i] = __uint_as_float(((uint32_t)(uint16_t)x[i]) << 16);
-    }
-  } else {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) v[i] = (k + i < k_limit) ? to_f32(p[i]) : 0.f;
-  }
-}
-
 template <typename TA, typename TW, typename TO>
 __global__ void __launch_bounds__(256) gemm_fma_kernel(const TA* __restrict__ a, const TW* __restrict__ w, const float* __restrict__ bias,
                                                        TO* __restrict__ out, int m, int n, int k, int a_vec, int w_vec) {

@@ -1,0 +1,197 @@
+// Kernels of attention over a cached latent, for gfx950.
+//
+//   latent_rotate_write: per token, the rotation of every head's rotated query part into the queries the attention
+//     kernels read, and (for a layer that makes its own latent) the RMS norm of the latent, the rotation of the shared key
+//     part and the write of both into the paged cache, as keys [page, 1, offset, D] and transposed as values
+//     [page, 1, D, offset].  All arithmetic is float32; values are rounded once, at the store.
+//   head_linear: one small product per head over the step's tokens, out[t, g] = maps[g] x[t, g], with heads at fixed
+//     strides inside the rows of x and out, and optionally a sigmoid gate as its epilogue.
+#include "common.h"
+
+// ---------------------------------------------------------------------------------------------
+// One block per token.  A row of `projected` holds [q: heads x (dim + rot) | ... | down: rank + rot at down_offset].
+//   queries[t, h, rank + c]       = rotated(q[t, h, dim + c]),  c < rot
+//   queries[t, h, rank + rot ..]  = 0 up to D (the first `rank` channels of a head are written by head_linear)
+//   down_offset >= 0:  cached[0 .. rank) = latent / sqrt(mean(latent^2) + eps) * norm_weight
+//                      cached[rank .. rank + rot) = rotated(shared key part), cached[rank + rot .. D) = 0
+// The rotation turns the first 2 * half channels of a rotated part and passes the rest: pairs are (2i, 2i + 1) when
+// `interleaved`, else (i, i + half); (u, v) -> (u cos - v sin, v cos + u sin) with cos/sin = table[position, i].
+// ---------------------------------------------------------------------------------------------
+__device__ __forceinline__ float rotated_channel(float own, float partner, bool is_first, float c, float s) {
+  return is_first ? own * c - partner * s : own * c + partner * s;
+}
+
+template <typename T>
+__device__ __forceinline__ float rotate_at(const T* __restrict__ part, int ch, int half, bool interleaved, const float* __restrict__ cs,
+                                           const float* __restrict__ sn) {
+  const float own = to_f32(part[ch]);
+  if (ch >= 2 * half) return own;
+  int i, partner;
+  bool first;
+  if (interleaved) { i = ch >> 1; partner = ch ^ 1; first = (ch & 1) == 0; }
+  else { first = ch < half; i = first ? ch : ch - half; partner = first ? ch + half : ch - half; }
+  return rotated_channel(own, to_f32(part[partner]), first, cs[i], sn[i]);
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256) latent_rotate_write_kernel(const T* __restrict__ projected, int width, T* __restrict__ queries, int heads, int dim,
+                                                                  int rot, int rank, int cached, int down_offset, const int* __restrict__ positions,
+                                                                  const float* __restrict__ cos_table, const float* __restrict__ sin_table, int half,
+                                                                  int interleaved, const float* __restrict__ norm_weight, float eps,
+                                                                  const int* __restrict__ slots, T* __restrict__ k_cache, T* __restrict__ v_cache,
+                                                                  int page_size) {
+  __shared__ float scratch[16];
+  const int t = blockIdx.x;
+  const T* row = projected + (size_t)t * width;
+  const int pos = positions[t];
+  const float* cs = half ? cos_table + (size_t)pos * half : nullptr;
+  const float* sn = half ? sin_table + (size_t)pos * half : nullptr;
+  const int tail = cached - rank;  // channels of a head's query behind the room for the mapped plain part
+  T* q_out = queries + (size_t)t * heads * cached;
+  for (int item = threadIdx.x; item < heads * tail; item += blockDim.x) {
+    const int h = item / tail, c = item % tail;
+    float v = 0.f;
+    if (c < rot) v = rotate_at<T>(row + h * (dim + rot) + dim, c, half, interleaved != 0, cs, sn);
+    q_out[h * cached + rank + c] = from_f32<T>(v);
+  }
+  if (down_offset < 0) return;  // (uniform over the block)
+  const T* down = row + down_offset;
+  float sumsq = 0.f;
+  for (int i = threadIdx.x; i < rank; i += blockDim.x) {
+    const float x = to_f32(down[i]);
+    sumsq += x * x;
+  }
+  const float inv = 1.0f / sqrtf(block_sum(sumsq, scratch) / (float)rank + eps);
+  const int slot = slots[t];
+  const size_t page = (size_t)(slot / page_size);
+  const int offset = slot % page_size;
+  T* k_dst = k_cache + (page * page_size + offset) * cached;
+  T* v_dst = v_cache + page * cached * page_size + offset;
+  for (int i = threadIdx.x; i < cached; i += blockDim.x) {
+    float v = 0.f;
+    if (i < rank) v = to_f32(down[i]) * inv * norm_weight[i];
+    else if (i < rank + rot) v = rotate_at<T>(down + rank, i - rank, half, interleaved != 0, cs, sn);
+    const T stored = from_f32<T>(v);
+    k_dst[i] = stored;
+    v_dst[(size_t)i * page_size] = stored;
+  }
+}
+
+extern "C" int velox_latent_rotate_write(const void* projected, int width, void* queries, int tokens, int heads, int dim, int rot, int rank, int cached,
+                                         int down_offset, const int* positions, const float* cos_table, const float* sin_table, int half, int interleaved,
+                                         const float* norm_weight, float eps, const int* slots, void* k_cache, void* v_cache, int page_size, int dtype,
+                                         hipStream_t stream) {
+  if (tokens <= 0) return 0;
+  if (heads < 1 || dim < 1 || rot < 0 || rank < 1 || cached < rank + rot || 2 * half > rot || page_size < 1) return -1;
+  if (heads * (dim + rot) > width || (down_offset >= 0 && (down_offset + rank + rot > width || norm_weight == nullptr))) return -1;
+  if (dtype == VELOX_BF16)
+    latent_rotate_write_kernel<bf16_t><<<tokens, 256, 0, stream>>>((const bf16_t*)projected, width, (bf16_t*)queries, heads, dim, rot, rank, cached, down_offset,
+                                                                   positions, cos_table, sin_table, half, interleaved, norm_weight, eps, slots,
+                                                                   (bf16_t*)k_cache, (bf16_t*)v_cache, page_size);
+  else
+    latent_rotate_write_kernel<float><<<tokens, 256, 0, stream>>>((const float*)projected, width, (float*)queries, heads, dim, rot, rank, cached, down_offset,
+                                                                  positions, cos_table, sin_table, half, interleaved, norm_weight, eps, slots,
+                                                                  (float*)k_cache, (float*)v_cache, page_size);
+  VELOX_RETURN_LAUNCH_STATUS();
+}
+
+// ---------------------------------------------------------------------------------------------
+// head_linear: out[t, g * out_stride + out_offset + j] = sum_k x[t, g * x_stride + x_offset + k] * maps[g, j, k]
+//   (* sigmoid(gate[t, gate_offset + g * n + j]) with a gate), for t < m, g < groups, j < n.
+// Exact float32 multiply-adds on 64 x 64 tiles through LDS, a head per blockIdx.z; every element is summed over k in one
+// fixed order by one thread, in inner sums of 128 terms (as the framework's float32 product does), so a row's result
+// depends on that row alone.
+// ---------------------------------------------------------------------------------------------
+#define HL_BM 64
+#define HL_BN 64
+#define HL_BK 16
+#define HL_PAD 4
+#define HL_FOLD 128
+
+template <typename T>
+__global__ void __launch_bounds__(256) head_linear_kernel(const T* __restrict__ x, int x_width, int x_stride, int x_offset, const T* __restrict__ maps,
+                                                          T* __restrict__ out, int out_width, int out_stride, int out_offset,
+                                                          const T* __restrict__ gate, int gate_width, int gate_offset, int m, int n, int k,
+                                                          int x_vec, int w_vec) {
+  __shared__ float a_tile[HL_BK][HL_BM + HL_PAD];
+  __shared__ float w_tile[HL_BK][HL_BN + HL_PAD];
+  const int g = blockIdx.z;
+  const int tid = threadIdx.x;
+  const int tx = tid % 16, ty = tid / 16;
+  const int m0 = blockIdx.y * HL_BM, n0 = blockIdx.x * HL_BN;
+  const int load_row = tid / 4, load_k = (tid % 4) * 4;
+  const bool a_row_ok = m0 + load_row < m;
+  const bool w_row_ok = n0 + load_row < n;
+  const size_t a_off = (size_t)(m0 + load_row) * x_width + (size_t)g * x_stride + x_offset;
+  const size_t w_off = ((size_t)g * n + n0 + load_row) * k;
+  float acc[4][4], total[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = total[i][j] = 0.f;
+  for (int k0 = 0; k0 < k; k0 += HL_BK) {
+    if (k0 % HL_FOLD == 0) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          total[i][j] += acc[i][j];
+          acc[i][j] = 0.f;
+        }
+    }
+    float av[4], wv[4];
+    load4<T>(x, a_off, k0 + load_k, k, a_row_ok, x_vec != 0, av);
+    load4<T>(maps, w_off, k0 + load_k, k, w_row_ok, w_vec != 0, wv);
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      a_tile[load_k + i][load_row] = av[i];
+      w_tile[load_k + i][load_row] = wv[i];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < HL_BK; ++kk) {
+      const float4_t ar = *reinterpret_cast<const float4_t*>(&a_tile[kk][ty * 4]);
+      const float4_t wr = *reinterpret_cast<const float4_t*>(&w_tile[kk][tx * 4]);
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(ar[i], wr[j], acc[i][j]);
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int row = m0 + ty * 4 + i;
+    if (row >= m) continue;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int col = n0 + tx * 4 + j;
+      if (col >= n) continue;
+      float v = total[i][j] + acc[i][j];
+      if (gate) {
+        const float z = to_f32(gate[(size_t)row * gate_width + gate_offset + g * n + col]);
+        v *= 1.f / (1.f + expf(-z));
+      }
+      out[(size_t)row * out_width + (size_t)g * out_stride + out_offset + col] = from_f32<T>(v);
+    }
+  }
+}
+
+extern "C" int velox_head_linear(const void* x, int x_width, int x_stride, int x_offset, const void* maps, void* out, int out_width, int out_stride,
+                                 int out_offset, const void* gate, int gate_width, int gate_offset, int m, int groups, int n, int k, int dtype,
+                                 hipStream_t stream) {
+  if (m <= 0 || groups <= 0 || n <= 0) return 0;
+  if (k < 1 || groups > 65535 || (groups - 1) * x_stride + x_offset + k > x_width || (groups - 1) * out_stride + out_offset + n > out_width) return -1;
+  if (gate != nullptr && gate_offset + groups * n > gate_width) return -1;
+  dim3 grid((n + HL_BN - 1) / HL_BN, (m + HL_BM - 1) / HL_BM, groups);
+  const int size = dtype == VELOX_BF16 ? 2 : 4;
+  const int x_vec = k % 4 == 0 && x_width % 4 == 0 && x_stride % 4 == 0 && x_offset % 4 == 0 && ((uintptr_t)x) % (4 * size) == 0;
+  const int w_vec = k % 4 == 0 && ((uintptr_t)maps) % (4 * size) == 0;
+  if (dtype == VELOX_BF16)
+    head_linear_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)x, x_width, x_stride, x_offset, (const bf16_t*)maps, (bf16_t*)out, out_width, out_stride,
+                                                         out_offset, (const bf16_t*)gate, gate_width, gate_offset, m, n, k, x_vec, w_vec);
+  else
+    head_linear_kernel<float><<<grid, 256, 0, stream>>>((const float*)x, x_width, x_stride, x_offset, (const float*)maps, (float*)out, out_width, out_stride,
+                                                        out_offset, (const float*)gate, gate_width, gate_offset, m, n, k, x_vec, w_vec);
+  VELOX_RETURN_LAUNCH_STATUS();
+}

@@ -1,0 +1,309 @@
+// Routed experts for gfx950: nothing about a step's routing is known to the host.
+//
+//   route_top:       scores of the router's float32 logits and the `top` largest per token
+//   routed_plan:     the step's (token, choice) pairs sorted by expert, and the list of row tiles that the grouped products
+//                    run: one workgroup, counters in LDS
+//   grouped_glu:     act[p, :] = silu(Wgate_e a_p) * (Wup_e a_p) for every sorted pair p of expert e, a_p = x[token of p]
+//                    (times the pair's weight when the weight scales the input)
+//   grouped_down:    y[p, :] = Wdown_e act[p, :] (times the pair's weight when it scales the output), float32
+//   routed_combine:  out[t, :] = sum_k y[place of pair (t, k), :] (+ shared[t, :]), the choices in order
+//
+// The grouped products are launched for the most tiles a step of its size can have; a workgroup beyond the step's own
+// number of tiles (read from the plan) exits at once.  A row's result is summed over k in one fixed order by one thread,
+// whatever other rows share its tile, so a token's output does not depend on which tokens go to the same experts or on
+// the order in which the plan's atomic counters placed them.
+#include "common.h"
+
+#define RT_BM 64  // rows of a tile (sorted pairs of one expert)
+#define RT_BN 64
+#define RT_BK 16
+#define RT_PAD 4
+#define RT_FOLD 128
+
+// ---------------------------------------------------------------------------------------------
+// route_top: one thread per token.  score = sigmoid(z) or softmax(z) over all experts; the `top` largest scores, ties to
+// the lower index; weights are the chosen scores, divided by their sum when `renormalize`.
+// ---------------------------------------------------------------------------------------------
+__global__ void __launch_bounds__(128) route_top_kernel(const float* __restrict__ logits, int* __restrict__ choice, float* __restrict__ weight, int tokens,
+                                                        int experts, int top, int softmax, int renormalize) {
+  const int t = blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= tokens) return;
+  const float* z = logits + (size_t)t * experts;
+  float shift = 0.f, denom = 1.f;
+  if (softmax) {
+    shift = z[0];
+    for (int e = 1; e < experts; ++e) shift = fmaxf(shift, z[e]);
+    denom = 0.f;
+    for (int e = 0; e < experts; ++e) denom += expf(z[e] - shift);
+  }
+  int* mine = choice + (size_t)t * top;
+  float* w = weight + (size_t)t * top;
+  float sum = 0.f;
+  for (int k = 0; k < top; ++k) {
+    int best = -1;
+    float best_score = 0.f;
+    for (int e = 0; e < experts; ++e) {
+      bool taken = false;
+      for (int j = 0; j < k; ++j) taken |= mine[j] == e;
+      if (taken) continue;
+      const float s = softmax ? expf(z[e] - shift) / denom : 1.f / (1.f + expf(-z[e]));
+      if (best < 0 || s > best_score) { best = e; best_score = s; }
+    }
+    mine[k] = best;
+    w[k] = best_score;
+    sum += best_score;
+  }
+  if (renormalize)
+    for (int k = 0; k < top; ++k) w[k] /= sum;
+}
+
+extern "C" int velox_route_top(const float* logits, int* choice, float* weight, int tokens, int experts, int top, int softmax, int renormalize,
+                               hipStream_t stream) {
+  if (tokens <= 0) return 0;
+  if (experts < 1 || top < 1 || top > experts) return -1;
+  route_top_kernel<<<(tokens + 127) / 128, 128, 0, stream>>>(logits, choice, weight, tokens, experts, top, softmax, renormalize);
+  VELOX_RETURN_LAUNCH_STATUS();
+}
+
+// ---------------------------------------------------------------------------------------------
+// The plan, int32: [0] number of tiles, [1 .. 1 + E] first sorted row of every expert and the total, then order[P]
+// (sorted row -> pair = token * top + k), place[P] (pair -> sorted row), tile_expert[max_tiles], tile_row[max_tiles].
+// ---------------------------------------------------------------------------------------------
+#define PLAN_MAX_EXPERTS 2048
+
+__global__ void __launch_bounds__(1024) routed_plan_kernel(const int* __restrict__ choice, int pairs, int experts, int max_tiles, int* __restrict__ plan) {
+  __shared__ int count[PLAN_MAX_EXPERTS];
+  __shared__ int first[PLAN_MAX_EXPERTS + 1];
+  int* num_tiles = plan;
+  int* starts = plan + 1;
+  int* order = starts + experts + 1;
+  int* place = order + pairs;
+  int* tile_expert = place + pairs;
+  int* tile_row = tile_expert + max_tiles;
+  for (int e = threadIdx.x; e < experts; e += blockDim.x) count[e] = 0;
+  __syncthreads();
+  for (int p = threadIdx.x; p < pairs; p += blockDim.x) {
+    const int e = choice[p];
+    if (e >= 0 && e < experts) atomicAdd(&count[e], 1);
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int at = 0, tiles = 0;
+    for (int e = 0; e < experts; ++e) {
+      first[e] = at;
+      starts[e] = at;
+      for (int r = 0; r < count[e] && tiles < max_tiles; r += RT_BM) {
+        tile_expert[tiles] = e;
+        tile_row[tiles] = at + r;
+        ++tiles;
+      }
+      at += count[e];
+      count[e] = 0;  // (from here on: how many of the expert's rows are placed)
+    }
+    first[experts] = at;
+    starts[experts] = at;
+    *num_tiles = tiles;
+  }
+  __syncthreads();
+  for (int p = threadIdx.x; p < pairs; p += blockDim.x) {
+    const int e = choice[p];
+    if (e < 0 || e >= experts) { place[p] = -1; continue; }
+    const int row = first[e] + atomicAdd(&count[e], 1);
+    order[row] = p;
+    place[p] = row;
+  }
+}
+
+extern "C" long long velox_routed_plan_elems(int pairs, int experts) {
+  const long long max_tiles = (pairs + RT_BM - 1) / RT_BM + experts;
+  return 1 + (experts + 1) + 2LL * pairs + 2 * max_tiles;
+}
+
+extern "C" int velox_routed_max_tiles(int pairs, int experts) { return (pairs + RT_BM - 1) / RT_BM + experts; }
+
+extern "C" int velox_routed_plan(const int* choice, int pairs, int experts, int* plan, hipStream_t stream) {
+  if (pairs <= 0) return 0;
+  if (experts < 1 || experts > PLAN_MAX_EXPERTS) return -1;
+  routed_plan_kernel<<<1, 1024, 0, stream>>>(choice, pairs, experts, velox_routed_max_tiles(pairs, experts), plan);
+  VELOX_RETURN_LAUNCH_STATUS();
+}
+
+// ---------------------------------------------------------------------------------------------
+// The grouped products.  GLU: two tiles of W (gate rows and the up rows of the same columns), the activation as the
+// epilogue.  Rows of A: GLU gathers x[token] (scaled by the pair's weight and rounded to T, as a product on T operands
+// would read it); the down product reads the sorted rows of act.
+// ---------------------------------------------------------------------------------------------
+template <typename T, typename TO, bool GLU>
+__global__ void __launch_bounds__(256) grouped_product_kernel(const T* __restrict__ a, const T* __restrict__ w, TO* __restrict__ out,
+                                                              const int* __restrict__ plan, const float* __restrict__ pair_weight, int pairs, int experts,
+                                                              int max_tiles, int top, int n, int k, int scale_rows, int a_vec, int w_vec) {
+  __shared__ float a_tile[RT_BK][RT_BM + RT_PAD];
+  __shared__ float w_tile[GLU ? 2 : 1][RT_BK][RT_BN + RT_PAD];
+  __shared__ int row_pair[RT_BM];
+  const int tile = blockIdx.y;
+  if (tile >= plan[0]) return;  // (uniform over the workgroup)
+  const int* starts = plan + 1;
+  const int* order = starts + experts + 1;
+  const int* tile_expert = order + 2 * (size_t)pairs;
+  const int* tile_row = tile_expert + max_tiles;
+  const int e = tile_expert[tile];
+  const int row0 = tile_row[tile];
+  const int rows = min(RT_BM, starts[e + 1] - row0);
+  const int tid = threadIdx.x;
+  const int tx = tid % 16, ty = tid / 16;
+  const int n0 = blockIdx.x * RT_BN;
+  const int load_row = tid / 4, load_k = (tid % 4) * 4;
+  if (tid < RT_BM) row_pair[tid] = tid < rows ? order[row0 + tid] : -1;
+  __syncthreads();
+  const bool a_row_ok = load_row < rows;
+  const int my_pair = row_pair[load_row];
+  size_t a_off = 0;
+  float a_scale = 1.f;
+  if (a_row_ok) {
+    if (GLU) {
+      a_off = (size_t)(my_pair / top) * k;
+      if (scale_rows) a_scale = pair_weight[my_pair];
+    } else {
+      a_off = (size_t)(row0 + load_row) * k;
+    }
+  }
+  const bool w_row_ok = n0 + load_row < n;
+  const size_t w_rows = GLU ? 2 * (size_t)n : (size_t)n;  // rows of one expert's matrix
+  const size_t w_off = ((size_t)e * w_rows + n0 + load_row) * k;
+  const size_t up_off = w_off + (size_t)n * k;
+
+  constexpr int NW = GLU ? 2 : 1;
+  float acc[NW][4][4], total[NW][4][4];
+#pragma unroll
+  for (int u = 0; u < NW; ++u)
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[u][i][j] = total[u][i][j] = 0.f;
+
+  for (int k0 = 0; k0 < k; k0 += RT_BK) {
+    if (k0 % RT_FOLD == 0) {
+#pragma unroll
+      for (int u = 0; u < NW; ++u)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            total[u][i][j] += acc[u][i][j];
+            acc[u][i][j] = 0.f;
+          }
+    }
+    float av[4], wv[NW][4];
+    load4<T>(a, a_off, k0 + load_k, k, a_row_ok, a_vec != 0, av);
+    if (GLU && scale_rows) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) av[i] = to_f32(from_f32<T>(av[i] * a_scale));
+    }
+    load4<T>(w, w_off, k0 + load_k, k, w_row_ok, w_vec != 0, wv[0]);
+    if (GLU) load4<T>(w, up_off, k0 + load_k, k, w_row_ok, w_vec != 0, wv[NW - 1]);
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      a_tile[load_k + i][load_row] = av[i];
+#pragma unroll
+      for (int u = 0; u < NW; ++u) w_tile[u][load_k + i][load_row] = wv[u][i];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < RT_BK; ++kk) {
+      const float4_t ar = *reinterpret_cast<const float4_t*>(&a_tile[kk][ty * 4]);
+#pragma unroll
+      for (int u = 0; u < NW; ++u) {
+        const float4_t wr = *reinterpret_cast<const float4_t*>(&w_tile[u][kk][tx * 4]);
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) acc[u][i][j] = fmaf(ar[i], wr[j], acc[u][i][j]);
+      }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = ty * 4 + i;
+    if (r >= rows) continue;
+    const float row_scale = (!GLU && scale_rows) ? pair_weight[row_pair[r]] : 1.f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int col = n0 + tx * 4 + j;
+      if (col >= n) continue;
+      float v = total[0][i][j] + acc[0][i][j];
+      if (GLU) {
+        const float up = total[NW - 1][i][j] + acc[NW - 1][i][j];
+        v = v / (1.f + expf(-v)) * up;  // (float32 throughout, one rounding at the store)
+      } else {
+        v *= row_scale;
+      }
+      out[(size_t)(row0 + r) * n + col] = from_f32<TO>(v);
+    }
+  }
+}
+
+extern "C" int velox_grouped_glu(const void* x, const void* gate_up, void* act, const int* plan, const float* pair_weight, int pairs, int experts, int top,
+                                 int inter, int hidden, int scale_input, int dtype, hipStream_t stream) {
+  if (pairs <= 0) return 0;
+  const int max_tiles = velox_routed_max_tiles(pairs, experts);
+  dim3 grid((inter + RT_BN - 1) / RT_BN, max_tiles);
+  if (grid.y > 65535) return -1;
+  const int size = dtype == VELOX_BF16 ? 2 : 4;
+  const int a_vec = hidden % 4 == 0 && ((uintptr_t)x) % (4 * size) == 0;
+  const int w_vec = hidden % 4 == 0 && ((uintptr_t)gate_up) % (4 * size) == 0;
+  if (dtype == VELOX_BF16)
+    grouped_product_kernel<bf16_t, bf16_t, true><<<grid, 256, 0, stream>>>((const bf16_t*)x, (const bf16_t*)gate_up, (bf16_t*)act, plan, pair_weight, pairs, experts,
+                                                                           max_tiles, top, inter, hidden, scale_input, a_vec, w_vec);
+  else
+    grouped_product_kernel<float, float, true><<<grid, 256, 0, stream>>>((const float*)x, (const float*)gate_up, (float*)act, plan, pair_weight, pairs, experts,
+                                                                         max_tiles, top, inter, hidden, scale_input, a_vec, w_vec);
+  VELOX_RETURN_LAUNCH_STATUS();
+}
+
+extern "C" int velox_grouped_down(const void* act, const void* down, float* y, const int* plan, const float* pair_weight, int pairs, int experts, int top,
+                                  int hidden, int inter, int scale_output, int dtype, hipStream_t stream) {
+  if (pairs <= 0) return 0;
+  const int max_tiles = velox_routed_max_tiles(pairs, experts);
+  dim3 grid((hidden + RT_BN - 1) / RT_BN, max_tiles);
+  if (grid.y > 65535) return -1;
+  const int size = dtype == VELOX_BF16 ? 2 : 4;
+  const int a_vec = inter % 4 == 0 && ((uintptr_t)act) % (4 * size) == 0;
+  const int w_vec = inter % 4 == 0 && ((uintptr_t)down) % (4 * size) == 0;
+  if (dtype == VELOX_BF16)
+    grouped_product_kernel<bf16_t, float, false><<<grid, 256, 0, stream>>>((const bf16_t*)act, (const bf16_t*)down, y, plan, pair_weight, pairs, experts, max_tiles,
+                                                                           top, hidden, inter, scale_output, a_vec, w_vec);
+  else
+    grouped_product_kernel<float, float, false><<<grid, 256, 0, stream>>>((const float*)act, (const float*)down, y, plan, pair_weight, pairs, experts, max_tiles,
+                                                                          top, hidden, inter, scale_output, a_vec, w_vec);
+  VELOX_RETURN_LAUNCH_STATUS();
+}
+
+// ---------------------------------------------------------------------------------------------
+// out[t, :] = (sum_k y[place[t * top + k], :]) + shared[t, :], the choices added in order, one rounding at the store.
+// ---------------------------------------------------------------------------------------------
+template <typename T>
+__global__ void __launch_bounds__(256) routed_combine_kernel(const float* __restrict__ y, const int* __restrict__ place, const T* __restrict__ shared,
+                                                             T* __restrict__ out, int top, int hidden) {
+  const int t = blockIdx.x;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    float v = 0.f;
+    for (int k = 0; k < top; ++k) {
+      const int row = place[(size_t)t * top + k];
+      if (row >= 0) v += y[(size_t)row * hidden + i];
+    }
+    if (shared) v += to_f32(shared[(size_t)t * hidden + i]);
+    out[(size_t)t * hidden + i] = from_f32<T>(v);
+  }
+}
+
+extern "C" int velox_routed_combine(const float* y, const int* plan, const void* shared, void* out, int tokens, int top, int experts, int hidden, int dtype,
+                                    hipStream_t stream) {
+  if (tokens <= 0) return 0;
+  const int* place = plan + 1 + (experts + 1) + (size_t)tokens * top;
+  if (dtype == VELOX_BF16)
+    routed_combine_kernel<bf16_t><<<tokens, 256, 0, stream>>>(y, place, (const bf16_t*)shared, (bf16_t*)out, top, hidden);
+  else
+    routed_combine_kernel<float><<<tokens, 256, 0, stream>>>(y, place, (const float*)shared, (float*)out, top, hidden);
+  VELOX_RETURN_LAUNCH_STATUS();
+}

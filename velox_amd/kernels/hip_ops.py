@@ -20,7 +20,7 @@ from typing import Tuple, Dict, Optional
 
 import torch
 
-from ..parts.base import DeferredNorm, ResidualSink
+from ..parts.base import DeferredNorm, ResidualSink, SumOf
 from . import build
 
 logger = logging.getLogger(__name__)
@@ -102,9 +102,9 @@ class HipOps:
     # -- loading --------------------------------------------------------------------------------
     def _declare_core(self) -> None:
         c = self._core
-        c.velox_embed.argtypes = [_P, _P, _P, _I, _I, _I, _I, _P]
+        c.velox_embed.argtypes = [_P, _P, _P, _I, _I, _I, _I, _F, _P]
         c.velox_place_tokens.argtypes = [_P, _P, _P, _P, _I, _I, _I, _P]
-        c.velox_add_rmsnorm.argtypes = [_P, _P, _P, _P, _P, _I, _I, _F, _I, _I, _I, ctypes.c_longlong, _P]
+        c.velox_add_rmsnorm.argtypes = [_P, _P, _P, _P, _P, _I, _I, _F, _I, _I, _I, ctypes.c_longlong, _P, _I, _P]
         c.velox_skinny_qkv_rotary_bf16.argtypes = [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P, _I, _F, _F, _I, _P]
         c.velox_silu_mul.argtypes = [_P, _P, _I, _I, _I, _P]
         c.velox_rope_kv_write.argtypes = [_P, _P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P]
@@ -137,6 +137,18 @@ class HipOps:
         c.velox_probe_mfma.restype = _I
         c.velox_probe_grid_barrier.argtypes = [_I, _I, _I, _P, _P, _P]
         c.velox_probe_grid_barrier.restype = _I
+        c.velox_latent_rotate_write.argtypes = [_P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _P, _P, _P, _I, _I, _P, _F, _P, _P, _P, _I, _I, _P]
+        c.velox_head_linear.argtypes = [_P, _I, _I, _I, _P, _P, _I, _I, _I, _P, _I, _I, _I, _I, _I, _I, _I, _P]
+        c.velox_route_top.argtypes = [_P, _P, _P, _I, _I, _I, _I, _I, _P]
+        c.velox_routed_plan_elems.argtypes = [_I, _I]
+        c.velox_routed_plan_elems.restype = ctypes.c_longlong
+        c.velox_routed_plan.argtypes = [_P, _I, _I, _P, _P]
+        c.velox_grouped_glu.argtypes = [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P]
+        c.velox_grouped_down.argtypes = [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P]
+        c.velox_routed_combine.argtypes = [_P, _P, _P, _P, _I, _I, _I, _I, _I, _P]
+        for fn in (c.velox_latent_rotate_write, c.velox_head_linear, c.velox_route_top, c.velox_routed_plan, c.velox_grouped_glu, c.velox_grouped_down,
+                   c.velox_routed_combine):
+            fn.restype = _I
         for fn in (c.velox_embed, c.velox_place_tokens, c.velox_add_rmsnorm, c.velox_silu_mul, c.velox_rope_kv_write, c.velox_gemm_fma,
                    c.velox_argmax, c.velox_sample, c.velox_sample_chunked, c.velox_apply_penalties, c.velox_count_tokens, c.velox_count_sampled,
                    c.velox_penalties_from_counts):
@@ -286,14 +298,14 @@ class HipOps:
             raise KernelError(f"{what}: launch failed with HIP error {status}")
 
     # -- embedding and norms ----------------------------------------------------------------------
-    def embed(self, token_ids: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
+    def embed(self, token_ids: torch.Tensor, table: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
         self._check("token_ids", token_ids, torch.int32)
         self._check("table", table)
         if token_ids.dim() != 1 or table.dim() != 2:
             raise KernelError("embed: token_ids must be [T] and the table [V, H]")
         vocab, hidden = table.shape
         out = torch.empty((token_ids.shape[0], hidden), dtype=torch.float32, device=self.device)
-        status = self._core.velox_embed(_ptr(token_ids), _ptr(table), _ptr(out), token_ids.shape[0], hidden, vocab, _code(table.dtype), self._stream())
+        status = self._core.velox_embed(_ptr(token_ids), _ptr(table), _ptr(out), token_ids.shape[0], hidden, vocab, _code(table.dtype), float(scale), self._stream())
         self._launched(status, "embed")
         return out
 
@@ -316,6 +328,10 @@ class HipOps:
         tokens, hidden = residual.shape
         self._check("weight", weight, torch.float32, (hidden,))
         partials, partial_stride = 1, 0
+        second = None
+        if isinstance(delta, SumOf):  # two terms, added to each other first
+            delta, second = delta.first, delta.second
+            self._check("second term of the delta", second, None, (tokens, hidden))
         if delta is not None:
             if delta.dim() == 3:  # partial sums of a split product, added here
                 partials, partial_stride = delta.shape[0], tokens * hidden
@@ -329,7 +345,8 @@ class HipOps:
             count = tokens
         out = torch.empty((count, hidden), dtype=out_dtype, device=self.device)
         delta_code = _code(delta.dtype) if delta is not None else _code(out_dtype)
-        status = self._core.velox_add_rmsnorm(_ptr(residual), _ptr(delta), _ptr(rows), _ptr(weight), _ptr(out), count, hidden, float(eps), delta_code, _code(out_dtype), partials, partial_stride, self._stream())
+        status = self._core.velox_add_rmsnorm(_ptr(residual), _ptr(delta), _ptr(rows), _ptr(weight), _ptr(out), count, hidden, float(eps), delta_code, _code(out_dtype), partials, partial_stride,
+                                              _ptr(second), _code(second.dtype) if second is not None else 0, self._stream())
         self._launched(status, "add_rmsnorm")
         return out
 
@@ -726,6 +743,118 @@ class HipOps:
             int(x_packed is not None), self._stream())
         self._launched(status, "skinny_qkv_rotary")
         return q
+
+    # -- attention over a cached latent -----------------------------------------------------------
+    def latent_rotate_write(self, projected, num_heads, dim, rot_dim, kv_rank, cached_dim, down_offset, positions, cos, sin, interleaved,
+                            norm_weight, eps, slot_mapping, k_cache, v_cache, block_size) -> torch.Tensor:
+        """Rows of ``projected`` hold ``num_heads`` queries of ``dim`` plain and ``rot_dim`` rotated channels and, at
+        ``down_offset`` (-1: none, nothing is written to the cache), a latent of ``kv_rank`` and a shared key part of
+        ``rot_dim`` channels.  Returns the queries the attention kernels read, ``[T, num_heads * cached_dim]``: of every head
+        the channels from ``kv_rank`` on are written here (the rotated part, then zeros), the first ``kv_rank`` are left
+        for ``head_linear``.  The normed latent and the rotated shared part go into the cache."""
+        if projected.dim() != 2:
+            raise KernelError("latent_rotate_write: rows are [T, width]")
+        tokens, width = projected.shape
+        self._check("projected", projected, None, (tokens, width))
+        self._check("positions", positions, torch.int32, (tokens,))
+        half = 0
+        if cos is not None:
+            self._check("cos", cos, torch.float32)
+            self._check("sin", sin, torch.float32, tuple(cos.shape))
+            half = cos.shape[1]
+        if (num_heads * (dim + rot_dim) > width or 2 * half > rot_dim or cached_dim < kv_rank + rot_dim
+                or (down_offset >= 0 and down_offset + kv_rank + rot_dim > width)):
+            raise KernelError(f"latent_rotate_write: rows of {width} do not hold {num_heads} x ({dim} + {rot_dim}) queries and a latent of {kv_rank} + {rot_dim} at {down_offset}")
+        if down_offset >= 0:
+            self._check("slot_mapping", slot_mapping, torch.int32, (tokens,))
+            self._check("norm_weight", norm_weight, torch.float32, (kv_rank,))
+            pages = k_cache.shape[0]
+            self._check("k_cache", k_cache, projected.dtype, (pages, 1, block_size, cached_dim))
+            self._check("v_cache", v_cache, projected.dtype, (pages, 1, cached_dim, block_size))
+        queries = torch.empty((tokens, num_heads * cached_dim), dtype=projected.dtype, device=self.device)
+        status = self._core.velox_latent_rotate_write(
+            _ptr(projected), width, _ptr(queries), tokens, num_heads, dim, rot_dim, kv_rank, cached_dim, int(down_offset), _ptr(positions), _ptr(cos), _ptr(sin),
+            half, int(bool(interleaved)), _ptr(norm_weight) if down_offset >= 0 else _P(0), float(eps), _ptr(slot_mapping) if down_offset >= 0 else _P(0),
+            _ptr(k_cache) if down_offset >= 0 else _P(0), _ptr(v_cache) if down_offset >= 0 else _P(0), int(block_size), _code(projected.dtype), self._stream())
+        self._launched(status, "latent_rotate_write")
+        return queries
+
+    def head_linear(self, x, x_head_stride, x_offset, maps, out, out_head_stride, out_offset, gate=None, gate_offset=0) -> torch.Tensor:
+        """``out[t, g * out_head_stride + out_offset + j] = sum_k x[t, g * x_head_stride + x_offset + k] * maps[g, j, k]``, times
+        ``sigmoid(gate[t, gate_offset + g * n + j])`` when ``gate`` is given: one small product per head, the heads at fixed
+        strides inside the rows of ``x`` and ``out`` (written in place, other columns untouched)."""
+        if x.dim() != 2 or out.dim() != 2 or maps.dim() != 3 or x.shape[0] != out.shape[0]:
+            raise KernelError("head_linear: x and out are [T, width], maps is [groups, n, k]")
+        groups, n, k = maps.shape
+        self._check("x", x)
+        self._check("maps", maps, x.dtype)
+        self._check("out", out, x.dtype)
+        if (min(x_head_stride, x_offset, out_head_stride, out_offset) < 0 or (groups - 1) * x_head_stride + x_offset + k > x.shape[1]
+                or (groups - 1) * out_head_stride + out_offset + n > out.shape[1]):
+            raise KernelError("head_linear: a head's channels lie outside the rows")
+        gate_width = 0
+        if gate is not None:
+            self._check("gate", gate, x.dtype)
+            gate_width = gate.shape[1]
+            if gate.dim() != 2 or gate.shape[0] != x.shape[0] or gate_offset < 0 or gate_offset + groups * n > gate_width:
+                raise KernelError("head_linear: the gate's columns lie outside its rows")
+        status = self._core.velox_head_linear(_ptr(x), x.shape[1], int(x_head_stride), int(x_offset), _ptr(maps), _ptr(out), out.shape[1], int(out_head_stride),
+                                              int(out_offset), _ptr(gate), gate_width, int(gate_offset), x.shape[0], groups, n, k, _code(x.dtype), self._stream())
+        self._launched(status, "head_linear")
+        return out
+
+    # -- routed experts ---------------------------------------------------------------------------
+    def route_top(self, logits: torch.Tensor, top: int, score: str = "sigmoid", renormalize: bool = False):
+        """float32 ``logits`` [T, E] -> (int32 choices [T, top], float32 weights [T, top]): the ``top`` largest scores
+        (``sigmoid`` or ``softmax`` over all experts), ties to the lower index, divided by their sum when ``renormalize``."""
+        self._check("logits", logits, torch.float32)
+        if logits.dim() != 2 or not 1 <= top <= logits.shape[1] or score not in ("sigmoid", "softmax"):
+            raise KernelError(f"route_top: logits {tuple(logits.shape)}, top={top}, score={score!r}")
+        tokens, experts = logits.shape
+        choice = torch.empty((tokens, top), dtype=torch.int32, device=self.device)
+        weight = torch.empty((tokens, top), dtype=torch.float32, device=self.device)
+        self._launched(self._core.velox_route_top(_ptr(logits), _ptr(choice), _ptr(weight), tokens, experts, int(top), int(score == "softmax"),
+                                                  int(bool(renormalize)), self._stream()), "route_top")
+        return choice, weight
+
+    def routed_plan_elems(self, max_num_tokens: int, top: int, experts: int) -> int:
+        """int32 elements of the plan of a step of at most ``max_num_tokens`` tokens."""
+        return int(self._core.velox_routed_plan_elems(int(max_num_tokens) * int(top), int(experts)))
+
+    def routed_experts(self, x, choice, weight, gate_up_weight, down_weight, num_experts: int, scale_input: bool, shared, out_dtype, workspace=None):
+        """``sum_k unit_{choice[t, k]}(weight[t, k] x[t])`` (or the weight on the unit's output), plus ``shared``: the pairs
+        are sorted by expert on the device, two grouped products run every expert on its rows, and each token's results
+        are added in the order of its choices.  ``gate_up_weight`` [E * 2F, H] (per expert gate rows, then up rows),
+        ``down_weight`` [E * H, F]."""
+        tokens, hidden = x.shape
+        top = choice.shape[1]
+        pairs = tokens * top
+        inter = gate_up_weight.shape[0] // (2 * num_experts)
+        self._check("x", x)
+        self._check("choice", choice, torch.int32, (tokens, top))
+        self._check("weight", weight, torch.float32, (tokens, top))
+        self._check("gate_up_weight", gate_up_weight, x.dtype, (num_experts * 2 * inter, hidden))
+        self._check("down_weight", down_weight, x.dtype, (num_experts * hidden, inter))
+        if shared is not None:
+            self._check("shared", shared, out_dtype, (tokens, hidden))
+        if out_dtype != x.dtype:
+            raise KernelError("routed_experts: the result has the activations' dtype")
+        elems = self.routed_plan_elems(tokens, top, num_experts)
+        if workspace is not None:
+            plan = workspace.get("routed_plan", elems).view(torch.int32)
+        else:
+            plan = torch.empty(elems, dtype=torch.int32, device=self.device)
+        self._launched(self._core.velox_routed_plan(_ptr(choice), pairs, num_experts, _ptr(plan), self._stream()), "routed_plan")
+        act = torch.empty((pairs, inter), dtype=x.dtype, device=self.device)
+        self._launched(self._core.velox_grouped_glu(_ptr(x), _ptr(gate_up_weight), _ptr(act), _ptr(plan), _ptr(weight), pairs, num_experts, top, inter, hidden,
+                                                    int(bool(scale_input)), _code(x.dtype), self._stream()), "grouped_glu")
+        y = torch.empty((pairs, hidden), dtype=torch.float32, device=self.device)
+        self._launched(self._core.velox_grouped_down(_ptr(act), _ptr(down_weight), _ptr(y), _ptr(plan), _ptr(weight), pairs, num_experts, top, hidden, inter,
+                                                     int(not scale_input), _code(x.dtype), self._stream()), "grouped_down")
+        out = torch.empty((tokens, hidden), dtype=out_dtype, device=self.device)
+        self._launched(self._core.velox_routed_combine(_ptr(y), _ptr(plan), _ptr(shared), _ptr(out), tokens, top, num_experts, hidden, _code(out_dtype),
+                                                       self._stream()), "routed_combine")
+        return out
 
     # -- attention ------------------------------------------------------------------------------
     def choose_splits(self, num_seqs: int, num_kv_heads: int, row_tiles: int, max_kv_len: int, all_decode: bool) -> int:

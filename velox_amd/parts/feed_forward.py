@@ -49,10 +49,10 @@ class GatedMLP(FeedForward):
     accepts_sink = True  # its last product may add itself to the residual (ResidualSink)
     accepts_deferred = True  # its first product can read a DeferredNorm
 
-    def forward(self, x, ctx, sink=None):
+    def forward(self, x, ctx, sink=None, partials_ok: bool = True):
         ops = ctx.ops
         act = ops.linear_silu_mul(x, self.operand("gate_up_weight"), ctx.dtype)
-        return ops.linear(act, self.operand("down_weight"), None, ctx.dtype, partials_ok=True, residual_norm=sink)
+        return ops.linear(act, self.operand("down_weight"), None, ctx.dtype, partials_ok=partials_ok, residual_norm=sink)
 
 
 register_part("feed_forward", "gated_mlp", GatedMLP)
@@ -131,9 +131,7 @@ class RoutedExperts(FeedForward):
         x = ops.materialize(x)
         logits = ops.linear(x, self.router_weight, None, torch.float32)
         choice, weight = ops.route_top(logits, self.top, self.score, self.renormalize)
-        shared = self.shared.forward(x, ctx) if self.shared is not None else None
-        if shared is not None and shared.dim() == 3:
-            shared = shared.sum(0)  # (partial sums of a split product; the experts' results are added to one tensor)
+        shared = self.shared.forward(x, ctx, partials_ok=False) if self.shared is not None else None
         return ops.routed_experts(x, choice, weight, self.gate_up_weight, self.down_weight, self.num_experts, self.scale_input, shared,
                                   ctx.dtype, ctx.workspace)
 
