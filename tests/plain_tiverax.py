@@ -140,7 +140,7 @@ def tiverax_logits(config: dict, weights: Dict[str, torch.Tensor], token_ids, dt
     ids = torch.as_tensor(list(token_ids), dtype=torch.long)
     positions = torch.arange(ids.shape[0])
     eps = float(config["norm"]["eps"])
-    x = w["embed"][ids] * float(config["embedding"]["scale"])
+    x = w["embed"][ids] * float((config.get("embedding") or {}).get("scale", 1.0))
     kept = {}
     for index, layer in enumerate(config["layers"]):
         if layer["type"] != "latent_attention":
