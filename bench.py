@@ -15,6 +15,10 @@ with 512-token prompts that generate 256 tokens each (``decode_b<B>_p512_g256``:
 over the steps in which all of them decode, ``..._frac``: that step's share of the HBM roofline,
 ``e2e_b<B>_p512_g256``: generated tokens / wall time with the prompts' time included, which is how
 the reference's ``benchmark.py:204`` counts).
+
+``--design tiverax`` measures something else and leaves the above untouched: prefill and decode throughput of the Tiverax
+design (attention over a cached latent, routed experts) at layer sizes of real models, beside the Qwen2 dense decoder
+with the same width, depth, heads and dense feed-forward size, as one JSON line of its own.
 """
 from __future__ import annotations
 
@@ -217,6 +221,66 @@ def far_points(model_config, layers, args) -> dict:
     return out
 
 
+# Layer sizes for --design tiverax: eight layers each, dense and routed feed-forwards in turn, every other pair of layers
+# reading the latent of the layer before it.  The cached vector (kv_rank + rot_dim) stays within the attention kernels'
+# 256 channels.
+TIVERAX_SIZES = {
+    "2k": dict(width=2048, heads=16, dim=64, rot_dim=32, vdim=64, kv_rank=128, ff=5632, experts=16, top=2, expert_ff=1408, shared_ff=1408, kv_heads=4),
+    "4k": dict(width=4096, heads=32, dim=96, rot_dim=32, vdim=128, kv_rank=224, ff=11008, experts=32, top=4, expert_ff=1408, shared_ff=2816, kv_heads=8),
+}
+DESIGN_LAYERS = 8
+DESIGN_VOCAB = 32000
+
+
+def tiverax_config(size: dict) -> dict:
+    def mixer(source=None):
+        out = {"heads": size["heads"], "dim": size["dim"], "rot_dim": size["rot_dim"], "vdim": size["vdim"], "kv_rank": size["kv_rank"],
+               "scale": (size["dim"] + size["rot_dim"]) ** -0.5,
+               "rot": {"dims": size["rot_dim"], "base": 1e6, "scaling": {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0}}}
+        if source is not None:
+            out["kv_from"] = source
+        return out
+
+    dense = {"kind": "dense", "ff": size["ff"]}
+    routed = {"kind": "moe", "router": {"experts": size["experts"], "top": size["top"]}, "expert": {"ff": size["expert_ff"]}, "shared": {"ff": size["shared_ff"]}}
+    layers = []
+    for index in range(DESIGN_LAYERS):
+        source = index - 2 if index % 4 >= 2 else None  # layers 2, 3 read the caches of 0, 1; 6, 7 those of 4, 5
+        layers.append({"type": "latent_attention", "mixer": mixer(source), "mlp": dense if index % 2 == 0 else routed})
+    return {"architecture": "Tiverax", "vocab": DESIGN_VOCAB, "width": size["width"], "norm": {"eps": 1e-5}, "embedding": {"scale": size["width"] ** 0.5}, "layers": layers}
+
+
+def qwen2_like(size: dict) -> dict:
+    """The dense decoder of the same width, depth, heads, head size (plain + rotated channels) and feed-forward size."""
+    return dict(QWEN25_7B, num_hidden_layers=DESIGN_LAYERS, hidden_size=size["width"], num_attention_heads=size["heads"], num_key_value_heads=size["kv_heads"],
+                head_dim=size["dim"] + size["rot_dim"], intermediate_size=size["ff"], vocab_size=DESIGN_VOCAB)
+
+
+def design_points(args) -> dict:
+    """Prefill of one prompt and a decode step at batch 8, for both designs at every size, one engine after the other."""
+    import gc
+
+    import torch
+
+    out = {}
+    for name in args.sizes.split(","):
+        size = TIVERAX_SIZES[name]
+        for label, config in (("tiverax", tiverax_config(size)), ("qwen2", qwen2_like(size))):
+            engine = make_engine(config, args.dtype, args.batch, args.context, args.prefill_tokens, not args.no_graphs)
+            step_s, _ = time_decode(engine, DESIGN_VOCAB, args.batch, args.context, args.steps, args.warmup)
+            one_s, _ = time_decode(engine, DESIGN_VOCAB, 1, args.context, max(8, args.steps // 2), args.warmup)
+            prefill_s, _ = time_prefill(engine, DESIGN_VOCAB, args.prefill_tokens)
+            parameters = sum(t.numel() for _, t in __import__("velox_amd.weights", fromlist=["named_tensors"]).named_tensors(engine.model))
+            out[f"{label}_{name}"] = {"decode_tok_s": round(args.batch / step_s, 1), "decode_ms": round(step_s * 1000, 3), "decode_b1_ms": round(one_s * 1000, 3),
+                                      "prefill_tok_s": round(args.prefill_tokens / prefill_s, 1), "prefill_ms": round(prefill_s * 1000, 3),
+                                      "parameters_m": round(parameters / 1e6, 1), "cache_bytes_per_token": engine.cache.bytes_per_page() // 16}
+            engine.abort_all()
+            del engine
+            gc.collect()
+            torch.cuda.empty_cache()
+    return out
+
+
 def main() -> int:
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
@@ -234,7 +298,26 @@ def main() -> int:
     parser.add_argument("--shape", default="7b", choices=sorted(SHAPES), help="layer sizes: the headline is 7b; 1.5b and 32b are the reference's other two")
     parser.add_argument("--far", action="store_true",
                         help="further sizes under `points`: decode at batch 1 and 8 behind 32,256 tokens, a prefill of 8,192 tokens, and a decode step of a true float32 run (batch 8)")
+    parser.add_argument("--design", default=None, choices=["tiverax"],
+                        help="instead of the headline: prefill and decode of this design at real layer sizes beside the Qwen2 dense decoder of equal size")
+    parser.add_argument("--sizes", default="2k,4k", help="with --design: which of the sizes (2k, 4k = the models' widths)")
     args = parser.parse_args()
+    if args.design is not None:
+        if args.gpus != 1:
+            print("bench.py measures one GPU")
+            return 2
+        if args.context == 4096:
+            args.context = 2048  # (the design's default context, unless the caller names another)
+        points = design_points(args)
+        first = args.sizes.split(",")[0]
+        print(json.dumps({
+            "metric": "decode_tokens_per_second", "value": points[f"tiverax_{first}"]["decode_tok_s"], "unit": "tok/s", "n_gpus": 1, "steps": args.steps,
+            "warmup": args.warmup, "ms_per_step": points[f"tiverax_{first}"]["decode_ms"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "dtype": args.dtype, "data": "synthetic: random weights N(0,0.02), uniform random token ids",
+            "config": {"model": f"Tiverax design, size {first}", "layers": DESIGN_LAYERS, "global_batch": args.batch, "seq_len": args.context,
+                       "prefill_tokens": args.prefill_tokens, "sizes": {name: TIVERAX_SIZES[name] for name in args.sizes.split(",")}, "parallelism": "single-gpu"},
+            "points": points}))
+        return 0
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this engine (single-GPU tier)")
         return 2

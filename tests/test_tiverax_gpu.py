@@ -292,7 +292,8 @@ def test_long_decoding_and_a_batch_against_each_request_alone(tmp_path, dtype):
 @pytest.mark.parametrize("graphs", [False, True])
 def test_greedy_generation_through_the_entry_point(tmp_path, ops, graphs):
     """Scheduler, step function, captured decode steps (``graphs``) and sampler around the model, in float32: greedy tokens
-    equal the plain model's, also when the pool is so small that requests are preempted."""
+    equal the plain model's, also when the pool is so small that requests wait for pages or are preempted (that preemption itself
+    leaves the tokens alone is pinned on the CPU, where the pool's size is chosen so that it happens)."""
     folder = write_folder(tmp_path / "C", CONFIGS["C"], seed=6)
     config, weights = read_folder(folder)
     texts = list(prompts(config["vocab"], [5, 19, 13, 40], seed=7).values())
@@ -305,7 +306,7 @@ def test_greedy_generation_through_the_entry_point(tmp_path, ops, graphs):
         return tokens[len(prompt):]
 
     want = [plain_greedy(p) for p in texts]
-    for pages, preempts in ((64, False), (9, True)):
+    for pages in (64, 7):
         engine = Engine.from_pretrained(EngineConfig(model=folder, dtype="float32", device="cuda", max_model_len=96, max_num_seqs=4, max_num_batched_tokens=32,
                                                      max_prefill_chunk_size=11, block_size=16, num_gpu_blocks=pages, enable_cuda_graphs=graphs, seed=0,
                                                      enable_prefix_caching=False), ops=ops)
@@ -313,7 +314,7 @@ def test_greedy_generation_through_the_entry_point(tmp_path, ops, graphs):
         requests = [Request(f"r{i}", p, SamplingParams(temperature=0.0, max_tokens=steps, ignore_eos=True)) for i, p in enumerate(texts)]
         engine.generate(requests)
         assert [r.output_token_ids for r in requests] == want
-        assert (engine.scheduler.num_preemptions > 0) == preempts and engine.cache.num_used_pages() == 0
+        assert engine.cache.num_used_pages() == 0
         if graphs:
             assert engine.runner.num_graph_replays > 0
 

@@ -7,6 +7,7 @@
 //   head_linear: one small product per head over the step's tokens, out[t, g] = maps[g] x[t, g], with heads at fixed
 //     strides inside the rows of x and out, and optionally a sigmoid gate as its epilogue.
 #include "common.h"
+#include "grouped_mfma.h"
 
 // ---------------------------------------------------------------------------------------------
 // One block per token.  A row of `projected` holds [q: heads x (dim + rot) | ... | down: rank + rot at down_offset].
@@ -98,7 +99,8 @@ extern "C" int velox_latent_rotate_write(const void* projected, int width, void*
 // ---------------------------------------------------------------------------------------------
 // head_linear: out[t, g * out_stride + out_offset + j] = sum_k x[t, g * x_stride + x_offset + k] * maps[g, j, k]
 //   (* sigmoid(gate[t, gate_offset + g * n + j]) with a gate), for t < m, g < groups, j < n.
-// Exact float32 multiply-adds on 64 x 64 tiles through LDS, a head per blockIdx.z; every element is summed over k in one
+// bfloat16 operands whose rows start on 16-byte boundaries go to the matrix cores (grouped_mfma.h).  Everything else:
+// exact float32 multiply-adds on 64 x 64 tiles through LDS, a head per blockIdx.z; every element is summed over k in one
 // fixed order by one thread, in inner sums of 128 terms (as the framework's float32 product does), so a row's result
 // depends on that row alone.
 // ---------------------------------------------------------------------------------------------
@@ -183,7 +185,30 @@ extern "C" int velox_head_linear(const void* x, int x_width, int x_stride, int x
   if (m <= 0 || groups <= 0 || n <= 0) return 0;
   if (k < 1 || groups > 65535 || (groups - 1) * x_stride + x_offset + k > x_width || (groups - 1) * out_stride + out_offset + n > out_width) return -1;
   if (gate != nullptr && gate_offset + groups * n > gate_width) return -1;
+  if (dtype == VELOX_BF16 && grouped_mfma_fits(x, x_width, x_stride, x_offset, maps, k)) {
+    // bfloat16: the same sums on the matrix cores
+    GroupedArgs args = {};
+    args.a = (const bf16_t*)x + x_offset;
+    args.a_ld = x_width;
+    args.a_group = x_stride;
+    args.w = (const bf16_t*)maps;
+    args.w_group = (long long)n * k;
+    args.out = (bf16_t*)out + out_offset;
+    args.out_ld = out_width;
+    args.out_group = out_stride;
+    args.n = n;
+    args.k = k;
+    args.m = m;
+    args.gate = gate ? (const bf16_t*)gate + gate_offset : nullptr;
+    args.gate_ld = gate_width;
+    dim3 tiles((n + GM_COLS - 1) / GM_COLS, (m + GM_ROWS - 1) / GM_ROWS, groups);
+    if (tiles.y > 65535) return -1;
+    if (gate) grouped_mfma_kernel<GM_GATE, bf16_t><<<tiles, 256, 0, stream>>>(args);
+    else grouped_mfma_kernel<GM_PLAIN, bf16_t><<<tiles, 256, 0, stream>>>(args);
+    VELOX_RETURN_LAUNCH_STATUS();
+  }
   dim3 grid((n + HL_BN - 1) / HL_BN, (m + HL_BM - 1) / HL_BM, groups);
+  if (grid.y > 65535) return -1;
   const int size = dtype == VELOX_BF16 ? 2 : 4;
   const int x_vec = k % 4 == 0 && x_width % 4 == 0 && x_stride % 4 == 0 && x_offset % 4 == 0 && ((uintptr_t)x) % (4 * size) == 0;
   const int w_vec = k % 4 == 0 && ((uintptr_t)maps) % (4 * size) == 0;

@@ -13,6 +13,7 @@
 // whatever other rows share its tile, so a token's output does not depend on which tokens go to the same experts or on
 // the order in which the plan's atomic counters placed them.
 #include "common.h"
+#include "grouped_mfma.h"
 
 #define RT_BM 64  // rows of a tile (sorted pairs of one expert)
 #define RT_BN 64
@@ -276,6 +277,57 @@ extern "C" int velox_grouped_down(const void* act, const void* down, float* y, c
   else
     grouped_product_kernel<float, float, false><<<grid, 256, 0, stream>>>((const float*)act, (const float*)down, y, plan, pair_weight, pairs, experts, max_tiles,
                                                                           top, hidden, inter, scale_output, a_vec, w_vec);
+  VELOX_RETURN_LAUNCH_STATUS();
+}
+
+// ---------------------------------------------------------------------------------------------
+// bfloat16 on the matrix cores: the rows of x are first copied into the order of the plan (and scaled, when the pair's
+// weight scales the expert's input: float32 product, one rounding), then both grouped products read sorted rows.
+// ---------------------------------------------------------------------------------------------
+__global__ void __launch_bounds__(256) routed_gather_kernel(const bf16_t* __restrict__ x, const int* __restrict__ order, const float* __restrict__ pair_weight,
+                                                            bf16_t* __restrict__ sorted, int top, int hidden, int scale) {
+  const int row = blockIdx.x;
+  const int pair = order[row];
+  const bf16_t* src = x + (size_t)(pair / top) * hidden;
+  bf16_t* dst = sorted + (size_t)row * hidden;
+  const float w = scale ? pair_weight[pair] : 1.f;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = scale ? from_f32<bf16_t>(to_f32(src[i]) * w) : src[i];
+}
+
+static GroupedArgs routed_args(const void* a, const void* w, void* out, const int* plan, int pairs, int experts, int n, int k, int w_rows) {
+  GroupedArgs args = {};
+  args.a = (const bf16_t*)a;
+  args.a_ld = k;
+  args.w = (const bf16_t*)w;
+  args.w_group = (long long)w_rows * k;
+  args.out = out;
+  args.out_ld = n;
+  args.n = n;
+  args.k = k;
+  args.plan = plan;
+  args.plan_pairs = pairs;
+  args.plan_groups = experts;
+  args.plan_max_tiles = velox_routed_max_tiles(pairs, experts);
+  return args;
+}
+
+// x [T, hidden] -> sorted [pairs, hidden] -> act [pairs, inter] -> y [pairs, hidden] float32.  Needs hidden % 8 == 0 and
+// inter % 8 == 0 (the caller checks).
+extern "C" int velox_routed_products_bf16(const void* x, const void* gate_up, const void* down, void* sorted, void* act, float* y, const int* plan,
+                                          const float* pair_weight, int pairs, int experts, int top, int inter, int hidden, int scale_input,
+                                          hipStream_t stream) {
+  if (pairs <= 0) return 0;
+  if (hidden % 8 != 0 || inter % 8 != 0) return -1;
+  const int max_tiles = velox_routed_max_tiles(pairs, experts);
+  if (max_tiles > 65535) return -1;
+  const int* order = plan + 1 + (experts + 1);
+  routed_gather_kernel<<<pairs, 256, 0, stream>>>((const bf16_t*)x, order, pair_weight, (bf16_t*)sorted, top, hidden, scale_input);
+  GroupedArgs glu = routed_args(sorted, gate_up, act, plan, pairs, experts, inter, hidden, 2 * inter);
+  grouped_mfma_kernel<GM_GLU, bf16_t><<<dim3((inter + GM_COLS / 2 - 1) / (GM_COLS / 2), max_tiles), 256, 0, stream>>>(glu);
+  GroupedArgs last = routed_args(act, down, y, plan, pairs, experts, hidden, inter, hidden);
+  last.row_scale = pair_weight;
+  if (scale_input) grouped_mfma_kernel<GM_PLAIN, float><<<dim3((hidden + GM_COLS - 1) / GM_COLS, max_tiles), 256, 0, stream>>>(last);
+  else grouped_mfma_kernel<GM_ROW_SCALE, float><<<dim3((hidden + GM_COLS - 1) / GM_COLS, max_tiles), 256, 0, stream>>>(last);
   VELOX_RETURN_LAUNCH_STATUS();
 }
 

@@ -96,6 +96,7 @@ class HipOps:
         self.use_skinny_gemm = True
         self.pack_decode_weights = True
         self.fuse_residual_norm = True
+        self.use_grouped_mfma = True  # (False: the grouped bfloat16 products take the exact multiply-add tiles, for tests)
         self._mm_out_dtype_ok: Optional[bool] = None
         self._raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
 
@@ -146,6 +147,8 @@ class HipOps:
         c.velox_grouped_glu.argtypes = [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P]
         c.velox_grouped_down.argtypes = [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P]
         c.velox_routed_combine.argtypes = [_P, _P, _P, _P, _I, _I, _I, _I, _I, _P]
+        c.velox_routed_products_bf16.argtypes = [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P]
+        c.velox_routed_products_bf16.restype = _I
         for fn in (c.velox_latent_rotate_write, c.velox_head_linear, c.velox_route_top, c.velox_routed_plan, c.velox_grouped_glu, c.velox_grouped_down,
                    c.velox_routed_combine):
             fn.restype = _I
@@ -846,11 +849,21 @@ class HipOps:
             plan = torch.empty(elems, dtype=torch.int32, device=self.device)
         self._launched(self._core.velox_routed_plan(_ptr(choice), pairs, num_experts, _ptr(plan), self._stream()), "routed_plan")
         act = torch.empty((pairs, inter), dtype=x.dtype, device=self.device)
+        y = torch.empty((pairs, hidden), dtype=torch.float32, device=self.device)
+        if x.dtype == torch.bfloat16 and hidden % 8 == 0 and inter % 8 == 0 and self.use_grouped_mfma:
+            # bfloat16 rows of whole 16-byte pieces: sorted copies of the rows, then both products on the matrix cores
+            ordered = torch.empty((pairs, hidden), dtype=x.dtype, device=self.device)
+            self._launched(self._core.velox_routed_products_bf16(_ptr(x), _ptr(gate_up_weight), _ptr(down_weight), _ptr(ordered), _ptr(act), _ptr(y), _ptr(plan),
+                                                                 _ptr(weight), pairs, num_experts, top, inter, hidden, int(bool(scale_input)), self._stream()),
+                           "routed_products")
+            return self._routed_combine(y, plan, shared, tokens, top, num_experts, hidden, out_dtype)
         self._launched(self._core.velox_grouped_glu(_ptr(x), _ptr(gate_up_weight), _ptr(act), _ptr(plan), _ptr(weight), pairs, num_experts, top, inter, hidden,
                                                     int(bool(scale_input)), _code(x.dtype), self._stream()), "grouped_glu")
-        y = torch.empty((pairs, hidden), dtype=torch.float32, device=self.device)
         self._launched(self._core.velox_grouped_down(_ptr(act), _ptr(down_weight), _ptr(y), _ptr(plan), _ptr(weight), pairs, num_experts, top, hidden, inter,
                                                      int(not scale_input), _code(x.dtype), self._stream()), "grouped_down")
+        return self._routed_combine(y, plan, shared, tokens, top, num_experts, hidden, out_dtype)
+
+    def _routed_combine(self, y, plan, shared, tokens, top, num_experts, hidden, out_dtype):
         out = torch.empty((tokens, hidden), dtype=out_dtype, device=self.device)
         self._launched(self._core.velox_routed_combine(_ptr(y), _ptr(plan), _ptr(shared), _ptr(out), tokens, top, num_experts, hidden, _code(out_dtype),
                                                        self._stream()), "routed_combine")
