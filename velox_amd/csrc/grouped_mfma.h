@@ -2,14 +2,16 @@
 // over its own rows, out[r, g, :] = W_g a[r, g, :].  Shared by the routed experts and by the per-head products of
 // attention over a latent.
 //
-// A workgroup of four waves owns 64 rows and 128 output columns of one group (64 gate and the 64 up columns of the same
-// outputs with the GLU epilogue); a wave owns 32 of the columns (two 16-row tiles of W; GLU: a gate tile and its up tile)
-// and all 64 rows, eight 16x16 accumulators.  Operands come straight from global memory in the layout of
-// v_mfma_f32_16x16x32_bf16 (lane = 16 g + i holds indices 8 g .. 8 g + 7 of row i: 16 bytes), W as the left operand, so
-// acc[j] of lane (g, i) is out[row i][column 4 g + j]; the next step's operands are asked for before this step's matrix
-// instructions.  The four waves read the same rows of `a`, which the compute unit's cache serves.  Rows and columns
-// beyond a tile's own read a valid row again and are never stored.  A row's sum is built in the order of k whatever
-// else is in the tile.
+// A workgroup of four waves owns 64 rows and 64 NT output columns of one group (NT = 2 or 4 tiles of W per wave; half as
+// many gate columns and the up columns of the same outputs with the GLU epilogue); a wave owns 16 NT of the columns and all
+// 64 rows: 4 NT 16x16 accumulators.  W comes straight from global memory in the layout of
+// v_mfma_f32_16x16x32_bf16 (lane = 16 g + i holds indices 8 g .. 8 g + 7 of row i: 16 bytes) and is the left operand, so
+// acc[j] of lane (g, i) is out[row i][column 4 g + j]; no two waves read the same W.  The rows of `a`, which all four
+// waves need, pass through LDS: a step is 64 indices, 8 KB for the 64 rows, two 16-byte pieces per thread, laid out [piece][row] so
+// that the 16 lanes of a lane group read 256 contiguous bytes (no bank conflicts on the reads, which are four times as many
+// as the writes); two buffers, one barrier per step, the
+// next step's pieces and W operands asked for before this step's matrix instructions.  Rows and columns beyond a tile's
+// own read a valid row again and are never stored.  A row's sum is built in the order of k whatever else is in the tile.
 //
 // Requirements (checked by the callers): K % 8 == 0, row strides and offsets of `a` multiples of 8 elements, 16-byte
 // aligned bases.
@@ -19,7 +21,7 @@
 typedef __bf16 gm_bf16x8_t __attribute__((ext_vector_type(8)));
 
 #define GM_ROWS 64       // rows of a tile
-#define GM_COLS 128      // output columns of a workgroup (GLU: 64)
+#define GM_FEW_COLS 32   // output columns of a workgroup of the kernel for few rows (GLU: 16)
 
 enum { GM_PLAIN = 0, GM_GLU = 1, GM_GATE = 2, GM_ROW_SCALE = 3 };
 
@@ -49,8 +51,10 @@ __device__ __forceinline__ gm_bf16x8_t gm_load(const bf16_t* p, bool ok) {
   return __builtin_bit_cast(gm_bf16x8_t, *reinterpret_cast<const float4_t*>(p));
 }
 
-template <int EPI, typename TO>
+template <int EPI, typename TO, int GM_NT>
 __global__ void __launch_bounds__(256) grouped_mfma_kernel(const GroupedArgs args) {
+  constexpr int GM_COLS = 64 * GM_NT;  // output columns of the workgroup (GLU: half as many)
+  __shared__ float4_t a_lds[2][2][256];
   int group, row0, rows;
   const int* order = nullptr;
   if (args.plan != nullptr) {
@@ -68,19 +72,128 @@ __global__ void __launch_bounds__(256) grouped_mfma_kernel(const GroupedArgs arg
     row0 = blockIdx.y * GM_ROWS;
     rows = min(GM_ROWS, args.m - row0);
   }
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int i = lane & 15, g4 = lane >> 4;
+  const int n = args.n, k = args.k;
+  // the tiles of W this wave owns: their first output columns (GLU: tiles 0, 1 are gate rows, 2, 3 the up rows of the same)
+  int col0[GM_NT];
+#pragma unroll
+  for (int t = 0; t < GM_NT; ++t) {
+    if (EPI == GM_GLU) col0[t] = blockIdx.x * (GM_COLS / 2) + wave * (8 * GM_NT) + (t % (GM_NT / 2)) * 16;
+    else col0[t] = blockIdx.x * GM_COLS + wave * (16 * GM_NT) + t * 16;
+  }
+  const bf16_t* w_base = args.w + (size_t)group * args.w_group;
+  const bf16_t* w_row[GM_NT];
+#pragma unroll
+  for (int t = 0; t < GM_NT; ++t) {
+    const int col = min(col0[t] + i, n - 1);
+    w_row[t] = w_base + (size_t)(EPI == GM_GLU && t >= GM_NT / 2 ? n + col : col) * k + 8 * g4;
+  }
+  // this thread's two pieces of the rows of `a`: row tid / 4, indices 8 (tid % 4) .. + 7 of each half of a step of 64
+  const bf16_t* a_piece = args.a + (size_t)(row0 + min(tid >> 2, rows - 1)) * args.a_ld + (size_t)group * args.a_group + 8 * (tid & 3);
+  float4_t acc[GM_NT][4];
+#pragma unroll
+  for (int t = 0; t < GM_NT; ++t)
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt) acc[t][mt] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+  gm_bf16x8_t w_cur[2][GM_NT], w_next[2][GM_NT];
+  const int a_slot = (tid & 3) * 64 + (tid >> 2);  // [piece][row]: a row tile's operand reads are then 256 contiguous bytes per 16 lanes
+#pragma unroll
+  for (int u = 0; u < 2; ++u) {
+#pragma unroll
+    for (int t = 0; t < GM_NT; ++t) w_cur[u][t] = gm_load(w_row[t] + 32 * u, 32 * u + 8 * g4 < k);
+    a_lds[0][u][a_slot] = __builtin_bit_cast(float4_t, gm_load(a_piece + 32 * u, 32 * u + 8 * (tid & 3) < k));
+  }
+  __syncthreads();
+  int buffer = 0;
+  for (int k0 = 0; k0 < k; k0 += 64) {
+    gm_bf16x8_t a_next[2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int at = k0 + 64 + 32 * u;
+#pragma unroll
+      for (int t = 0; t < GM_NT; ++t) w_next[u][t] = gm_load(w_row[t] + at, at + 8 * g4 < k);
+      a_next[u] = gm_load(a_piece + at, at + 8 * (tid & 3) < k);
+    }
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      gm_bf16x8_t a_cur[4];
+#pragma unroll
+      for (int mt = 0; mt < 4; ++mt) a_cur[mt] = __builtin_bit_cast(gm_bf16x8_t, a_lds[buffer][u][g4 * 64 + mt * 16 + i]);
+#pragma unroll
+      for (int t = 0; t < GM_NT; ++t)
+#pragma unroll
+        for (int mt = 0; mt < 4; ++mt) acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_cur[u][t], a_cur[mt], acc[t][mt], 0, 0, 0);
+    }
+#pragma unroll
+    for (int u = 0; u < 2; ++u) a_lds[buffer ^ 1][u][a_slot] = __builtin_bit_cast(float4_t, a_next[u]);
+    __syncthreads();
+    buffer ^= 1;
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int t = 0; t < GM_NT; ++t) w_cur[u][t] = w_next[u][t];
+  }
+
+  TO* out = reinterpret_cast<TO*>(args.out);
+#pragma unroll
+  for (int mt = 0; mt < 4; ++mt) {
+    const int r = mt * 16 + i;
+    if (r >= rows) continue;
+    const size_t out_row = (size_t)(row0 + r) * args.out_ld + (size_t)group * args.out_group;
+    float scale = 1.f;
+    if (EPI == GM_ROW_SCALE) scale = args.row_scale[order[row0 + r]];
+#pragma unroll
+    for (int t = 0; t < (EPI == GM_GLU ? GM_NT / 2 : GM_NT); ++t)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int col = col0[t] + 4 * g4 + j;
+        if (col >= n) continue;
+        float v = acc[t][mt][j];
+        if (EPI == GM_GLU) v = v / (1.f + expf(-v)) * acc[t + GM_NT / 2][mt][j];
+        if (EPI == GM_GATE) {
+          const float z = to_f32(args.gate[(size_t)(row0 + r) * args.gate_ld + (size_t)group * n + col]);
+          v *= 1.f / (1.f + expf(-z));
+        }
+        if (EPI == GM_ROW_SCALE) v *= scale;
+        out[out_row + col] = from_f32<TO>(v);
+      }
+  }
+}
+
+
+// The same products when no tile has more than 16 MT rows (a decode step's pairs): then a product is bound by reading W
+// once, and what counts is how many loads are in flight.  A workgroup owns 32 output columns (GLU: 16 gate columns and
+// their up columns) of one tile; its four waves split K into quarters, each wave asks for four steps' operands at once,
+// and the waves' sums are added through LDS in the order of the waves (no atomics: the same result on every run).
+template <int EPI, typename TO, int MT>
+__global__ void __launch_bounds__(256) grouped_mfma_few_rows_kernel(const GroupedArgs args) {
+  __shared__ float4_t partial[3][2 * MT][64];
+  int group, row0, rows;
+  const int* order = nullptr;
+  if (args.plan != nullptr) {
+    const int tile = blockIdx.y;
+    if (tile >= args.plan[0]) return;  // (uniform over the workgroup)
+    const int* starts = args.plan + 1;
+    order = starts + args.plan_groups + 1;
+    const int* tile_group = order + 2 * (size_t)args.plan_pairs;
+    const int* tile_row = tile_group + args.plan_max_tiles;
+    group = tile_group[tile];
+    row0 = tile_row[tile];
+    rows = min(16 * MT, starts[group + 1] - row0);
+  } else {
+    group = blockIdx.z;
+    row0 = blockIdx.y * 16 * MT;
+    rows = min(16 * MT, args.m - row0);
+  }
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int i = lane & 15, g4 = lane >> 4;
   const int n = args.n, k = args.k;
-  // the two tiles of W this wave owns: their first columns
   int col0[2];
-  if (EPI == GM_GLU) {
-    col0[0] = blockIdx.x * (GM_COLS / 2) + wave * 16;
-    col0[1] = col0[0];
-  } else {
-    col0[0] = blockIdx.x * GM_COLS + wave * 32;
-    col0[1] = col0[0] + 16;
-  }
-  if (col0[0] >= n) return;  // (a wave without columns; no barrier follows)
+  col0[0] = blockIdx.x * (EPI == GM_GLU ? GM_FEW_COLS / 2 : GM_FEW_COLS);
+  col0[1] = EPI == GM_GLU ? col0[0] : col0[0] + 16;
   const bf16_t* w_base = args.w + (size_t)group * args.w_group;
   const bf16_t* w_row[2];
 #pragma unroll
@@ -88,43 +201,54 @@ __global__ void __launch_bounds__(256) grouped_mfma_kernel(const GroupedArgs arg
     const int col = min(col0[t] + i, n - 1);
     w_row[t] = w_base + (size_t)(EPI == GM_GLU && t == 1 ? n + col : col) * k + 8 * g4;
   }
-  const bf16_t* a_row[4];
+  const bf16_t* a_row[MT];
 #pragma unroll
-  for (int mt = 0; mt < 4; ++mt) {
-    const int r = min(mt * 16 + i, rows - 1);
-    a_row[mt] = args.a + (size_t)(row0 + r) * args.a_ld + (size_t)group * args.a_group + 8 * g4;
-  }
-  float4_t acc[2][4];
+  for (int mt = 0; mt < MT; ++mt) a_row[mt] = args.a + (size_t)(row0 + min(mt * 16 + i, rows - 1)) * args.a_ld + (size_t)group * args.a_group + 8 * g4;
+  const int quarter = ((k + 127) / 128) * 32;  // indices per wave: a multiple of 32
+  const int k_begin = wave * quarter, k_end = min(k, k_begin + quarter);
+  float4_t acc[2][MT];
 #pragma unroll
   for (int t = 0; t < 2; ++t)
 #pragma unroll
-    for (int mt = 0; mt < 4; ++mt) acc[t][mt] = float4_t{0.f, 0.f, 0.f, 0.f};
-
-  gm_bf16x8_t w_cur[2], a_cur[4], w_next[2], a_next[4];
-  bool ok = 8 * g4 < k;
+    for (int mt = 0; mt < MT; ++mt) acc[t][mt] = float4_t{0.f, 0.f, 0.f, 0.f};
+  for (int k0 = k_begin; k0 < k_end; k0 += 128) {
+    gm_bf16x8_t wv[2][4], av[MT][4];
 #pragma unroll
-  for (int t = 0; t < 2; ++t) w_cur[t] = gm_load(w_row[t], ok);
+    for (int u = 0; u < 4; ++u) {
+      const bool ok = k0 + 32 * u + 8 * g4 < k_end;
 #pragma unroll
-  for (int mt = 0; mt < 4; ++mt) a_cur[mt] = gm_load(a_row[mt], ok);
-  for (int k0 = 0; k0 < k; k0 += 32) {
-    const bool more = k0 + 32 + 8 * g4 < k;
+      for (int t = 0; t < 2; ++t) wv[t][u] = gm_load(w_row[t] + k0 + 32 * u, ok);
 #pragma unroll
-    for (int t = 0; t < 2; ++t) w_next[t] = gm_load(w_row[t] + k0 + 32, more);
+      for (int mt = 0; mt < MT; ++mt) av[mt][u] = gm_load(a_row[mt] + k0 + 32 * u, ok);
+    }
 #pragma unroll
-    for (int mt = 0; mt < 4; ++mt) a_next[mt] = gm_load(a_row[mt] + k0 + 32, more);
+    for (int u = 0; u < 4; ++u)
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv[t][u], av[mt][u], acc[t][mt], 0, 0, 0);
+  }
+  if (wave > 0) {
 #pragma unroll
     for (int t = 0; t < 2; ++t)
 #pragma unroll
-      for (int mt = 0; mt < 4; ++mt) acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_cur[t], a_cur[mt], acc[t][mt], 0, 0, 0);
-#pragma unroll
-    for (int t = 0; t < 2; ++t) w_cur[t] = w_next[t];
-#pragma unroll
-    for (int mt = 0; mt < 4; ++mt) a_cur[mt] = a_next[mt];
+      for (int mt = 0; mt < MT; ++mt) partial[wave - 1][t * MT + mt][lane] = acc[t][mt];
   }
-
+  __syncthreads();
+  if (wave > 0) return;
+#pragma unroll
+  for (int other = 0; other < 3; ++other)
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        const float4_t p = partial[other][t * MT + mt][lane];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[t][mt][j] += p[j];
+      }
   TO* out = reinterpret_cast<TO*>(args.out);
 #pragma unroll
-  for (int mt = 0; mt < 4; ++mt) {
+  for (int mt = 0; mt < MT; ++mt) {
     const int r = mt * 16 + i;
     if (r >= rows) continue;
     const size_t out_row = (size_t)(row0 + r) * args.out_ld + (size_t)group * args.out_group;
@@ -148,7 +272,30 @@ __global__ void __launch_bounds__(256) grouped_mfma_kernel(const GroupedArgs arg
   }
 }
 
-// Whether the operands meet what the kernel's 16-byte loads need.
+// Launches the kernel that fits: `most_rows` is the most rows any tile can have (the plan's pairs, or m), `tiles_y` and
+// `tiles_z` the launch's other two dimensions.
+template <int EPI, typename TO>
+static void grouped_mfma_launch(const GroupedArgs& args, int most_rows, int tiles_y, int tiles_z, hipStream_t stream) {
+  const int n = args.n;
+  if (most_rows <= 64 && args.plan != nullptr) {
+    // (only with a plan: its tiles hold at most `most_rows` rows whatever their size; without one, rows come in tiles of the kernel's own size)
+    dim3 grid((n + (EPI == GM_GLU ? GM_FEW_COLS / 2 : GM_FEW_COLS) - 1) / (EPI == GM_GLU ? GM_FEW_COLS / 2 : GM_FEW_COLS), tiles_y, tiles_z);
+    if (most_rows <= 16) grouped_mfma_few_rows_kernel<EPI, TO, 1><<<grid, 256, 0, stream>>>(args);
+    else if (most_rows <= 32) grouped_mfma_few_rows_kernel<EPI, TO, 2><<<grid, 256, 0, stream>>>(args);
+    else grouped_mfma_few_rows_kernel<EPI, TO, 4><<<grid, 256, 0, stream>>>(args);
+    return;
+  }
+  const int outputs = EPI == GM_GLU ? 2 * n : n;  // rows of W
+  if (outputs <= 128) {
+    const int cols = EPI == GM_GLU ? 64 : 128;
+    grouped_mfma_kernel<EPI, TO, 2><<<dim3((n + cols - 1) / cols, tiles_y, tiles_z), 256, 0, stream>>>(args);
+  } else {
+    const int cols = EPI == GM_GLU ? 128 : 256;
+    grouped_mfma_kernel<EPI, TO, 4><<<dim3((n + cols - 1) / cols, tiles_y, tiles_z), 256, 0, stream>>>(args);
+  }
+}
+
+// Whether the operands meet what the kernels' 16-byte loads need.
 static inline bool grouped_mfma_fits(const void* a, long long a_ld, long long a_group, long long a_offset, const void* w, int k) {
   return k % 8 == 0 && a_ld % 8 == 0 && a_group % 8 == 0 && a_offset % 8 == 0 && ((uintptr_t)a) % 16 == 0 && ((uintptr_t)w) % 16 == 0;
 }

@@ -323,11 +323,11 @@ extern "C" int velox_routed_products_bf16(const void* x, const void* gate_up, co
   const int* order = plan + 1 + (experts + 1);
   routed_gather_kernel<<<pairs, 256, 0, stream>>>((const bf16_t*)x, order, pair_weight, (bf16_t*)sorted, top, hidden, scale_input);
   GroupedArgs glu = routed_args(sorted, gate_up, act, plan, pairs, experts, inter, hidden, 2 * inter);
-  grouped_mfma_kernel<GM_GLU, bf16_t><<<dim3((inter + GM_COLS / 2 - 1) / (GM_COLS / 2), max_tiles), 256, 0, stream>>>(glu);
+  grouped_mfma_launch<GM_GLU, bf16_t>(glu, pairs, max_tiles, 1, stream);
   GroupedArgs last = routed_args(act, down, y, plan, pairs, experts, hidden, inter, hidden);
   last.row_scale = pair_weight;
-  if (scale_input) grouped_mfma_kernel<GM_PLAIN, float><<<dim3((hidden + GM_COLS - 1) / GM_COLS, max_tiles), 256, 0, stream>>>(last);
-  else grouped_mfma_kernel<GM_ROW_SCALE, float><<<dim3((hidden + GM_COLS - 1) / GM_COLS, max_tiles), 256, 0, stream>>>(last);
+  if (scale_input) grouped_mfma_launch<GM_PLAIN, float>(last, pairs, max_tiles, 1, stream);
+  else grouped_mfma_launch<GM_ROW_SCALE, float>(last, pairs, max_tiles, 1, stream);
   VELOX_RETURN_LAUNCH_STATUS();
 }
 
