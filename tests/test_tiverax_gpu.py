@@ -228,7 +228,7 @@ def test_a_key_far_back_or_at_a_page_border_takes_the_attention(ops, far_at, len
 # the whole model
 # ----------------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
 def test_all_ways_of_cutting_on_the_gpu(tmp_path, name, dtype):
     folder = write_folder(tmp_path / name, CONFIGS[name], seed=2, dtype=dtype)
     config, weights = read_folder(folder)

@@ -70,8 +70,16 @@ CONFIG_C = {
         layer(mixer(2, 64, 32, 64, 96, 0.1), dense(128)),
     ],
 }
-CONFIGS = {"A": CONFIG_A, "B": CONFIG_B, "C": CONFIG_C}
-PAGE_SIZE = {"A": 4, "B": 8, "C": 16}
+# Nothing a multiple of 4, 8 or 16: rows of 200 bytes, odd heads, a cached vector of 24 channels, three experts of twelve.
+CONFIG_D = {
+    "architecture": "Tiverax", "vocab": 77, "width": 100, "norm": {"eps": 1e-5}, "embedding": {"scale": 0.5},
+    "layers": [
+        layer(mixer(3, 10, 6, 14, 18, 0.3, base=50.0, scaling=(3.0, 16, 4.0, 0.5)), moe(3, 2, 12, shared=20)),
+        layer(mixer(5, 6, 6, 2, 18, 0.4, base=50.0, scaling=(3.0, 16, 4.0, 0.5), kv_from=0), dense(36)),
+    ],
+}
+CONFIGS = {"A": CONFIG_A, "B": CONFIG_B, "C": CONFIG_C, "D": CONFIG_D}
+PAGE_SIZE = {"A": 4, "B": 8, "C": 16, "D": 16}
 
 
 def tensor_shapes(config: dict) -> Dict[str, tuple]:
