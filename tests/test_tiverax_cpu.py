@@ -91,7 +91,7 @@ def test_rotation_tables_hold_the_stretched_frequencies_and_the_magnitude(dims, 
     assert torch.equal(got[..., dims:], x[..., dims:])
 
 
-@pytest.mark.parametrize("name", ["A", "B", "D"])
+@pytest.mark.parametrize("name", ["A", "B", "D", "E"])
 def test_all_ways_of_cutting_agree_with_the_plain_model(tmp_path, name):
     """Whole prompts; the last tokens one by one; portions of 1 to 16 tokens (many of two); up to four requests mixed in
     a pool so small that pages and slots are used again; requests that are ended half way and recomputed."""

@@ -174,6 +174,26 @@ def test_routed_experts_part_against_the_design(ops):
     torch.testing.assert_close(got.cpu(), routed_experts(x, w, "f.", mlp), rtol=2e-4, atol=2e-5)
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("nh,nkv,d,window", [(4, 1, 272, None), (6, 2, 320, None), (2, 2, 1024, 37)])
+def test_attention_for_head_sizes_beyond_the_tiled_kernels(ops, dtype, nh, nkv, d, window):
+    """Head sizes above 256 go to the plain kernel: portions behind a context, single tokens and a first token in one step."""
+    ref, dt = TorchOps(), DTYPES[dtype]
+    page, pages = 8, 40
+    k_cache = torch.randn(pages, nkv, page, d).to(dt).cuda()
+    v_cache = torch.randn(pages, nkv, d, page).to(dt).cuda()
+    q_lens, kv_lens = [1, 1, 9, 1, 30], [70, 1, 9, 300, 155]  # (a decoded token behind 299 keys: two rounds of 256 keys)
+    tables = torch.zeros(5, 38, dtype=torch.int32)
+    perm = torch.randperm(pages - 1) + 1
+    tables[0, :9], tables[1, :1], tables[2, :2], tables[4, :20] = perm[:9], perm[9:10], perm[10:12], perm[12:32]
+    tables[3, :38] = torch.cat([perm[32:], perm[:31]])  # (this one shares pages with the others: only read here)
+    cu = torch.tensor([0, 1, 2, 11, 12, 42], dtype=torch.int32).cuda()
+    q = (torch.randn(42, nh * d) * 0.5).to(dt).cuda()
+    args = (q, nh, nkv, d, k_cache, v_cache, page, tables.cuda(), cu, torch.tensor(kv_lens, dtype=torch.int32).cuda(), 30, 300, 1.0 / math.sqrt(d), window, False, None)
+    got, want = ops.paged_attention(*args), ref.paged_attention(*args)
+    close(got, want, dtype)
+
+
 # ----------------------------------------------------------------------------------------------------
 # the mixer alone: one key made to stand out
 # ----------------------------------------------------------------------------------------------------
@@ -228,7 +248,7 @@ def test_a_key_far_back_or_at_a_page_border_takes_the_attention(ops, far_at, len
 # the whole model
 # ----------------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D", "E"])
 def test_all_ways_of_cutting_on_the_gpu(tmp_path, name, dtype):
     folder = write_folder(tmp_path / name, CONFIGS[name], seed=2, dtype=dtype)
     config, weights = read_folder(folder)

@@ -78,8 +78,16 @@ CONFIG_D = {
         layer(mixer(5, 6, 6, 2, 18, 0.4, base=50.0, scaling=(3.0, 16, 4.0, 0.5), kv_from=0), dense(36)),
     ],
 }
-CONFIGS = {"A": CONFIG_A, "B": CONFIG_B, "C": CONFIG_C, "D": CONFIG_D}
-PAGE_SIZE = {"A": 4, "B": 8, "C": 16, "D": 16}
+# A latent so wide that the cached vector (260 + 12 channels) is beyond the tiled attention kernels' 256.
+CONFIG_E = {
+    "architecture": "Tiverax", "vocab": 90, "width": 64, "norm": {"eps": 1e-5}, "embedding": {"scale": 2.0},
+    "layers": [
+        layer(mixer(2, 8, 12, 8, 260, 0.3, base=1000.0), dense(48)),
+        layer(mixer(3, 4, 12, 4, 260, 0.3, base=1000.0, kv_from=0), None),
+    ],
+}
+CONFIGS = {"A": CONFIG_A, "B": CONFIG_B, "C": CONFIG_C, "D": CONFIG_D, "E": CONFIG_E}
+PAGE_SIZE = {"A": 4, "B": 8, "C": 16, "D": 16, "E": 8}
 
 
 def tensor_shapes(config: dict) -> Dict[str, tuple]:

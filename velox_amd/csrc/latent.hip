@@ -220,3 +220,101 @@ extern "C" int velox_head_linear(const void* x, int x_width, int x_stride, int x
                                                         out_offset, (const float*)gate, gate_width, gate_offset, m, n, k, x_vec, w_vec);
   VELOX_RETURN_LAUNCH_STATUS();
 }
+
+// ---------------------------------------------------------------------------------------------
+// Attention over the paged cache for head sizes beyond the tiled kernels' 256 channels (any size up to 1,024): one
+// workgroup per (token, head), plain float32 arithmetic.  Keys [page, kv_head, offset, d], values transposed
+// [page, kv_head, d, offset].  256 keys at a time: a thread takes one key's score (the query sits in LDS), the workgroup
+// takes the maximum and the sum, and then every thread adds the 256 weighted values of its own channels; a running
+// maximum rescales what was added before.  Probabilities stay float32.
+// ---------------------------------------------------------------------------------------------
+#define PLAIN_ATTENTION_MAX_D 1024
+
+__device__ __forceinline__ float block_max_256(float v, float* scratch) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  v = wave_max(v);
+  __syncthreads();
+  if (lane == 0) scratch[wave] = v;
+  __syncthreads();
+  return fmaxf(fmaxf(scratch[0], scratch[1]), fmaxf(scratch[2], scratch[3]));
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256) plain_attention_kernel(const T* __restrict__ q, int q_width, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
+                                                              const int* __restrict__ block_tables, int table_width, const int* __restrict__ cu_q,
+                                                              const int* __restrict__ kv_lens, T* __restrict__ out, int num_seqs, int nh, int nkv, int d,
+                                                              int page_shift, float scale, int window) {
+  __shared__ float q_s[PLAIN_ATTENTION_MAX_D];
+  __shared__ float p_s[256];
+  __shared__ float scratch[16];
+  __shared__ int seq_s;
+  const int token = blockIdx.x, head = blockIdx.y, tid = threadIdx.x;
+  if (tid == 0) {
+    int b = 0;
+    while (b + 1 < num_seqs && cu_q[b + 1] <= token) ++b;
+    seq_s = b;
+  }
+  for (int c = tid; c < d; c += 256) q_s[c] = to_f32(q[(size_t)token * q_width + (size_t)head * d + c]);
+  __syncthreads();
+  const int b = seq_s;
+  const int kv_len = kv_lens[b];
+  const int last = kv_len - (cu_q[b + 1] - cu_q[b]) + (token - cu_q[b]);  // this token's position: the last key it sees
+  const int first = window > 0 ? max(0, last - window + 1) : 0;
+  const int kvh = head / (nh / nkv);
+  const int page_size = 1 << page_shift;
+  const int* table = block_tables + (size_t)b * table_width;
+  float running_max = -INFINITY, denom = 0.f;
+  float acc[PLAIN_ATTENTION_MAX_D / 256];
+#pragma unroll
+  for (int u = 0; u < PLAIN_ATTENTION_MAX_D / 256; ++u) acc[u] = 0.f;
+  for (int j0 = first; j0 <= last; j0 += 256) {
+    const int j = j0 + tid;
+    float s = -INFINITY;
+    if (j <= last) {
+      const T* key = k_cache + (((size_t)table[j >> page_shift] * nkv + kvh) * page_size + (j & (page_size - 1))) * d;
+      float dot = 0.f;
+      for (int c = 0; c < d; ++c) dot = fmaf(q_s[c], to_f32(key[c]), dot);
+      s = dot * scale;
+    }
+    const float new_max = fmaxf(running_max, block_max_256(s, scratch));  // (finite: key j0 is always seen)
+    const float p = j <= last ? expf(s - new_max) : 0.f;
+    p_s[tid] = p;
+    const float chunk_sum = block_sum(p, scratch);  // (its barriers also publish p_s)
+    const float alpha = expf(running_max - new_max);
+    denom = denom * alpha + chunk_sum;
+    running_max = new_max;
+    const int count = min(256, last - j0 + 1);
+#pragma unroll
+    for (int u = 0; u < PLAIN_ATTENTION_MAX_D / 256; ++u) {
+      const int c = tid + 256 * u;
+      if (c >= d) break;
+      float sum = 0.f;
+      for (int jj = 0; jj < count; ++jj) {
+        const int key = j0 + jj;
+        sum = fmaf(p_s[jj], to_f32(v_cache[(((size_t)table[key >> page_shift] * nkv + kvh) * d + c) * page_size + (key & (page_size - 1))]), sum);
+      }
+      acc[u] = acc[u] * alpha + sum;
+    }
+    __syncthreads();  // (p_s is written again in the next round)
+  }
+#pragma unroll
+  for (int u = 0; u < PLAIN_ATTENTION_MAX_D / 256; ++u) {
+    const int c = tid + 256 * u;
+    if (c < d) out[(size_t)token * nh * d + (size_t)head * d + c] = from_f32<T>(acc[u] / denom);
+  }
+}
+
+extern "C" int velox_plain_attention(const void* q, int q_width, const void* k_cache, const void* v_cache, const int* block_tables, int table_width,
+                                     const int* cu_q, const int* kv_lens, void* out, int num_seqs, int tokens, int nh, int nkv, int d, int page_shift,
+                                     float scale, int window, int dtype, hipStream_t stream) {
+  if (tokens <= 0) return 0;
+  if (d < 1 || d > PLAIN_ATTENTION_MAX_D || nh < 1 || nkv < 1 || nh % nkv != 0 || nh > 65535 || num_seqs < 1 || nh * d > q_width) return -1;
+  dim3 grid(tokens, nh);
+  if (dtype == VELOX_BF16)
+    plain_attention_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)q, q_width, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables, table_width,
+                                                             cu_q, kv_lens, (bf16_t*)out, num_seqs, nh, nkv, d, page_shift, scale, window);
+  else
+    plain_attention_kernel<float><<<grid, 256, 0, stream>>>((const float*)q, q_width, (const float*)k_cache, (const float*)v_cache, block_tables, table_width,
+                                                            cu_q, kv_lens, (float*)out, num_seqs, nh, nkv, d, page_shift, scale, window);
+  VELOX_RETURN_LAUNCH_STATUS();
+}

@@ -78,6 +78,7 @@ def _weight_of(weight) -> Tuple[torch.Tensor, Optional[PreparedWeight]]:
 
 class HipOps:
     name = "hip-gfx950"
+    MAX_TILED_HEAD_DIM = 256  # head sizes above this go to the plain attention kernel
 
     def __init__(self, device) -> None:
         self.device = torch.device(device)
@@ -140,6 +141,8 @@ class HipOps:
         c.velox_probe_grid_barrier.restype = _I
         c.velox_latent_rotate_write.argtypes = [_P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _P, _P, _P, _I, _I, _P, _F, _P, _P, _P, _I, _I, _P]
         c.velox_head_linear.argtypes = [_P, _I, _I, _I, _P, _P, _I, _I, _I, _P, _I, _I, _I, _I, _I, _I, _I, _P]
+        c.velox_plain_attention.argtypes = [_P, _I, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _P]
+        c.velox_plain_attention.restype = _I
         c.velox_route_top.argtypes = [_P, _P, _P, _I, _I, _I, _I, _I, _P]
         c.velox_routed_plan_elems.argtypes = [_I, _I]
         c.velox_routed_plan_elems.restype = ctypes.c_longlong
@@ -903,6 +906,8 @@ class HipOps:
         with the splits that ``choose_splits`` and ``choose_portion_splits`` pick.  The bound counts TOKENS, not sequences:
         the sequence on the null page that pads a step up to a timed number of rows (one more than ``max_num_seqs``) brings
         tokens within ``max_num_tokens`` like any other and is covered."""
+        if head_dim > self.MAX_TILED_HEAD_DIM:
+            return 0, 0  # (the plain kernel splits nothing)
         group = num_heads // num_kv_heads
         rows = 0  # splits x the rows the partial results are counted by
         for count in range(1, max_num_seqs + 1):  # single tokens, alone or before portions
@@ -946,9 +951,18 @@ class HipOps:
             raise KernelError(f"max_q_len={max_q_len} outside [1, {tokens}]")
         if not 0 <= decode_prefix <= num_seqs or num_seqs > tokens:
             raise KernelError(f"decode_prefix={decode_prefix} does not fit {num_seqs} sequences with {tokens} tokens")
+        out = torch.empty((tokens, num_heads * head_dim), dtype=qkv.dtype, device=self.device)
+        if head_dim > self.MAX_TILED_HEAD_DIM:
+            # beyond the tiled kernels: one workgroup per token and head, plain float32 arithmetic
+            if head_dim > 1024:
+                raise KernelError(f"paged_attention: head_dim={head_dim} is beyond every kernel (1,024 at most)")
+            status = self._core.velox_plain_attention(_ptr(qkv), width, _ptr(k_cache), _ptr(v_cache), _ptr(block_tables), block_tables.shape[1], _ptr(cu_q),
+                                                      _ptr(kv_lens), _ptr(out), num_seqs, tokens, num_heads, num_kv_heads, head_dim,
+                                                      block_size.bit_length() - 1, float(scale), int(window or 0), _code(qkv.dtype), self._stream())
+            self._launched(status, "plain_attention")
+            return out
         lib = self.attention_library(head_dim)
         group = num_heads // num_kv_heads
-        out = torch.empty((tokens, num_heads * head_dim), dtype=qkv.dtype, device=self.device)
 
         def launch(first_seq: int, count: int, first_token: int, num_tokens: int, longest: int, decode_only: bool, splits: Optional[int]) -> None:
             # sequences [first_seq, first_seq + count); their tokens are rows [first_token, first_token + num_tokens) of qkv

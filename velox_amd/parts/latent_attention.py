@@ -14,7 +14,8 @@ once (a product per head over the step's tokens only), the paged attention kerne
 whose "values" are the cached vectors themselves, and the result is taken through ``V_h``.  The cache is read as it
 stands, whatever the number of heads; keys and values per head are never formed.
 
-The cached vector is padded with zeros to a multiple of 16 channels (the attention kernels' tile), and is held
+The cached vector is padded with zeros to a multiple of 16 channels (the attention kernels' tile; beyond 256 channels a
+plain kernel of any size takes their place), and is held
 twice, as keys ``[page, 1, offset, D]`` and transposed as values ``[page, 1, D, offset]``, the layout those
 kernels read (``parts.attention.kv_pages``).
 
@@ -56,8 +57,8 @@ class LatentAttentionMixer(Mixer):
         self.names = dict(_NAMES)
         self.names.update(dict(names))
         self.cached_dim = (self.kv_rank + self.rot_dim + 15) // 16 * 16
-        if self.cached_dim > 256:
-            raise ValueError(f"kv_rank + rot_dim = {self.kv_rank + self.rot_dim}: the attention kernels take at most 256 cached channels per token")
+        if self.cached_dim > 1024:
+            raise ValueError(f"kv_rank + rot_dim = {self.kv_rank + self.rot_dim}: the attention kernels take at most 1,024 cached channels per token")
         self.q_size = self.num_heads * (self.dim + self.rot_dim)
         self.gate_size = self.num_heads * self.vdim if self.gate else 0
         self.down_size = self.kv_rank + self.rot_dim if self.own_latent else 0
@@ -103,8 +104,8 @@ class LatentAttentionMixer(Mixer):
 
     def prepare_kernels(self, ops) -> None:
         load = getattr(ops, "attention_library", None)
-        if load is not None:
-            load(self.cached_dim)
+        if load is not None and self.cached_dim <= getattr(ops, "MAX_TILED_HEAD_DIM", self.cached_dim):
+            load(self.cached_dim)  # (larger cached vectors go to the plain attention kernel of the core library)
         cos, _, _ = self._rotary()
         if cos is not None and 2 * cos.shape[1] > self.rot_dim:
             raise ValueError(f"the rotation spans {2 * cos.shape[1]} channels but the rotated part has {self.rot_dim}")
@@ -113,7 +114,7 @@ class LatentAttentionMixer(Mixer):
 
     def capture_key_bounds(self, ops, batch: int, max_model_len: int):
         choose = getattr(ops, "choose_splits", None)
-        if choose is None or max_model_len <= SHORT_CONTEXT_KEYS:
+        if choose is None or max_model_len <= SHORT_CONTEXT_KEYS or self.cached_dim > getattr(ops, "MAX_TILED_HEAD_DIM", self.cached_dim):
             return ()
         differs = choose(batch, 1, 1, max_model_len, True) != choose(batch, 1, 1, SHORT_CONTEXT_KEYS, True)
         return (SHORT_CONTEXT_KEYS,) if differs else ()
