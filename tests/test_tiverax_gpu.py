@@ -128,7 +128,8 @@ def test_router_scores_and_choices(ops, score, renormalize):
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("tokens,hidden,inter,experts,top,scale_input,with_shared", [(70, 64, 32, 4, 2, True, True), (9, 88, 20, 6, 3, True, False), (300, 96, 40, 8, 1, False, True),
-                                                                                   (1, 320, 96, 8, 1, True, True), (150, 72, 130, 3, 2, False, False)])
+                                                                                   (1, 320, 96, 8, 1, True, True), (150, 72, 130, 3, 2, False, False),
+                                                                                   (700, 136, 72, 2, 2, True, True), (900, 192, 80, 3, 1, False, False)])
 def test_routed_experts_against_the_plain_loop(ops, dtype, tokens, hidden, inter, experts, top, scale_input, with_shared):
     ref, dt = TorchOps(), DTYPES[dtype]
     x = torch.randn(tokens, hidden).to(dt).cuda()

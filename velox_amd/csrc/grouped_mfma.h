@@ -2,7 +2,7 @@
 // over its own rows, out[r, g, :] = W_g a[r, g, :].  Shared by the routed experts and by the per-head products of
 // attention over a latent.
 //
-// A workgroup of four waves owns 64 rows and 64 NT output columns of one group (NT = 2 or 4 tiles of W per wave; half as
+// A workgroup of four waves owns 64 rows (128 for the large tiles of a plan) and 64 NT output columns of one group (NT = 2 or 4 tiles of W per wave; half as
 // many gate columns and the up columns of the same outputs with the GLU epilogue); a wave owns 16 NT of the columns and all
 // 64 rows: 4 NT 16x16 accumulators.  W comes straight from global memory in the layout of
 // v_mfma_f32_16x16x32_bf16 (lane = 16 g + i holds indices 8 g .. 8 g + 7 of row i: 16 bytes) and is the left operand, so
@@ -20,7 +20,7 @@
 
 typedef __bf16 gm_bf16x8_t __attribute__((ext_vector_type(8)));
 
-#define GM_ROWS 64       // rows of a tile
+#define GM_ROWS 64       // rows of a tile without a plan (a plan's tiles hold 64 or 128)
 #define GM_FEW_COLS 32   // output columns of a workgroup of the kernel for few rows (GLU: 16)
 
 enum { GM_PLAIN = 0, GM_GLU = 1, GM_GATE = 2, GM_ROW_SCALE = 3 };
@@ -51,10 +51,14 @@ __device__ __forceinline__ gm_bf16x8_t gm_load(const bf16_t* p, bool ok) {
   return __builtin_bit_cast(gm_bf16x8_t, *reinterpret_cast<const float4_t*>(p));
 }
 
-template <int EPI, typename TO, int GM_NT>
+template <int EPI, typename TO, int GM_NT, int MT>
 __global__ void __launch_bounds__(256) grouped_mfma_kernel(const GroupedArgs args) {
-  constexpr int GM_COLS = 64 * GM_NT;  // output columns of the workgroup (GLU: half as many)
-  __shared__ float4_t a_lds[2][2][256];
+  constexpr int GM_COLS = 64 * GM_NT;    // output columns of the workgroup (GLU: half as many)
+  constexpr int ROWS = 16 * MT;          // rows of a tile: 64 or 128
+  constexpr int HALVES = MT == 8 ? 1 : 2;  // 32-index halves per step (the larger tile takes shorter steps: registers)
+  constexpr int STEP = 32 * HALVES;
+  constexpr int PIECES = MT / 4;         // 16-byte pieces of `a` per thread and half
+  __shared__ float4_t a_lds[2][HALVES][4 * ROWS];
   int group, row0, rows;
   const int* order = nullptr;
   if (args.plan != nullptr) {
@@ -66,17 +70,17 @@ __global__ void __launch_bounds__(256) grouped_mfma_kernel(const GroupedArgs arg
     const int* tile_row = tile_group + args.plan_max_tiles;
     group = tile_group[tile];
     row0 = tile_row[tile];
-    rows = min(GM_ROWS, starts[group + 1] - row0);
+    rows = min(ROWS, starts[group + 1] - row0);
   } else {
     group = blockIdx.z;
-    row0 = blockIdx.y * GM_ROWS;
-    rows = min(GM_ROWS, args.m - row0);
+    row0 = blockIdx.y * ROWS;
+    rows = min(ROWS, args.m - row0);
   }
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int i = lane & 15, g4 = lane >> 4;
   const int n = args.n, k = args.k;
-  // the tiles of W this wave owns: their first output columns (GLU: tiles 0, 1 are gate rows, 2, 3 the up rows of the same)
+  // the tiles of W this wave owns: their first output columns (GLU: the first half are gate rows, the others the up rows of the same)
   int col0[GM_NT];
 #pragma unroll
   for (int t = 0; t < GM_NT; ++t) {
@@ -90,56 +94,71 @@ __global__ void __launch_bounds__(256) grouped_mfma_kernel(const GroupedArgs arg
     const int col = min(col0[t] + i, n - 1);
     w_row[t] = w_base + (size_t)(EPI == GM_GLU && t >= GM_NT / 2 ? n + col : col) * k + 8 * g4;
   }
-  // this thread's two pieces of the rows of `a`: row tid / 4, indices 8 (tid % 4) .. + 7 of each half of a step of 64
-  const bf16_t* a_piece = args.a + (size_t)(row0 + min(tid >> 2, rows - 1)) * args.a_ld + (size_t)group * args.a_group + 8 * (tid & 3);
-  float4_t acc[GM_NT][4];
+  // this thread's pieces of the rows of `a`: piece q = tid + 256 p is row q / 4, indices 8 (q % 4) .. + 7 of a half; in LDS
+  // [part][row], so that a row tile's operand reads are 256 contiguous bytes per 16 lanes
+  const bf16_t* a_piece[PIECES];
+  int a_slot[PIECES];
+#pragma unroll
+  for (int p = 0; p < PIECES; ++p) {
+    const int q = tid + 256 * p;
+    a_piece[p] = args.a + (size_t)(row0 + min(q >> 2, rows - 1)) * args.a_ld + (size_t)group * args.a_group + 8 * (q & 3);
+    a_slot[p] = (q & 3) * ROWS + (q >> 2);
+  }
+  const int a_part = 8 * (tid & 3);  // (q % 4 is tid % 4 for every piece)
+  float4_t acc[GM_NT][MT];
 #pragma unroll
   for (int t = 0; t < GM_NT; ++t)
 #pragma unroll
-    for (int mt = 0; mt < 4; ++mt) acc[t][mt] = float4_t{0.f, 0.f, 0.f, 0.f};
+    for (int mt = 0; mt < MT; ++mt) acc[t][mt] = float4_t{0.f, 0.f, 0.f, 0.f};
 
-  gm_bf16x8_t w_cur[2][GM_NT], w_next[2][GM_NT];
-  const int a_slot = (tid & 3) * 64 + (tid >> 2);  // [piece][row]: a row tile's operand reads are then 256 contiguous bytes per 16 lanes
+  gm_bf16x8_t w_cur[HALVES][GM_NT], w_next[HALVES][GM_NT];
 #pragma unroll
-  for (int u = 0; u < 2; ++u) {
+  for (int u = 0; u < HALVES; ++u) {
 #pragma unroll
     for (int t = 0; t < GM_NT; ++t) w_cur[u][t] = gm_load(w_row[t] + 32 * u, 32 * u + 8 * g4 < k);
-    a_lds[0][u][a_slot] = __builtin_bit_cast(float4_t, gm_load(a_piece + 32 * u, 32 * u + 8 * (tid & 3) < k));
+#pragma unroll
+    for (int p = 0; p < PIECES; ++p) a_lds[0][u][a_slot[p]] = __builtin_bit_cast(float4_t, gm_load(a_piece[p] + 32 * u, 32 * u + a_part < k));
   }
   __syncthreads();
   int buffer = 0;
-  for (int k0 = 0; k0 < k; k0 += 64) {
-    gm_bf16x8_t a_next[2];
+  for (int k0 = 0; k0 < k; k0 += STEP) {
+    gm_bf16x8_t a_next[HALVES][PIECES];
 #pragma unroll
-    for (int u = 0; u < 2; ++u) {
-      const int at = k0 + 64 + 32 * u;
+    for (int u = 0; u < HALVES; ++u) {
+      const int at = k0 + STEP + 32 * u;
 #pragma unroll
       for (int t = 0; t < GM_NT; ++t) w_next[u][t] = gm_load(w_row[t] + at, at + 8 * g4 < k);
-      a_next[u] = gm_load(a_piece + at, at + 8 * (tid & 3) < k);
+#pragma unroll
+      for (int p = 0; p < PIECES; ++p) a_next[u][p] = gm_load(a_piece[p] + at, at + a_part < k);
     }
 #pragma unroll
-    for (int u = 0; u < 2; ++u) {
-      gm_bf16x8_t a_cur[4];
+    for (int u = 0; u < HALVES; ++u) {
 #pragma unroll
-      for (int mt = 0; mt < 4; ++mt) a_cur[mt] = __builtin_bit_cast(gm_bf16x8_t, a_lds[buffer][u][g4 * 64 + mt * 16 + i]);
+      for (int mh = 0; mh < MT; mh += 4) {  // four row tiles at a time: their operands live in registers together
+        gm_bf16x8_t a_cur[4];
 #pragma unroll
-      for (int t = 0; t < GM_NT; ++t)
+        for (int mt = 0; mt < 4; ++mt) a_cur[mt] = __builtin_bit_cast(gm_bf16x8_t, a_lds[buffer][u][g4 * ROWS + (mh + mt) * 16 + i]);
 #pragma unroll
-        for (int mt = 0; mt < 4; ++mt) acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_cur[u][t], a_cur[mt], acc[t][mt], 0, 0, 0);
+        for (int t = 0; t < GM_NT; ++t)
+#pragma unroll
+          for (int mt = 0; mt < 4; ++mt) acc[t][mh + mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_cur[u][t], a_cur[mt], acc[t][mh + mt], 0, 0, 0);
+      }
     }
 #pragma unroll
-    for (int u = 0; u < 2; ++u) a_lds[buffer ^ 1][u][a_slot] = __builtin_bit_cast(float4_t, a_next[u]);
+    for (int u = 0; u < HALVES; ++u)
+#pragma unroll
+      for (int p = 0; p < PIECES; ++p) a_lds[buffer ^ 1][u][a_slot[p]] = __builtin_bit_cast(float4_t, a_next[u][p]);
     __syncthreads();
     buffer ^= 1;
 #pragma unroll
-    for (int u = 0; u < 2; ++u)
+    for (int u = 0; u < HALVES; ++u)
 #pragma unroll
       for (int t = 0; t < GM_NT; ++t) w_cur[u][t] = w_next[u][t];
   }
 
   TO* out = reinterpret_cast<TO*>(args.out);
 #pragma unroll
-  for (int mt = 0; mt < 4; ++mt) {
+  for (int mt = 0; mt < MT; ++mt) {
     const int r = mt * 16 + i;
     if (r >= rows) continue;
     const size_t out_row = (size_t)(row0 + r) * args.out_ld + (size_t)group * args.out_group;
@@ -162,7 +181,6 @@ __global__ void __launch_bounds__(256) grouped_mfma_kernel(const GroupedArgs arg
       }
   }
 }
-
 
 // The same products when no tile has more than 16 MT rows (a decode step's pairs): then a product is bound by reading W
 // once, and what counts is how many loads are in flight.  A workgroup owns 32 output columns (GLU: 16 gate columns and
@@ -272,10 +290,11 @@ __global__ void __launch_bounds__(256) grouped_mfma_few_rows_kernel(const Groupe
   }
 }
 
-// Launches the kernel that fits: `most_rows` is the most rows any tile can have (the plan's pairs, or m), `tiles_y` and
-// `tiles_z` the launch's other two dimensions.
+// Launches the kernel that fits: `most_rows` is the most rows any tile can have (the plan's pairs, or m), `tile_rows` the
+// rows of the plan's tiles (64 or 128; without a plan rows come in tiles of 64), `tiles_y` and `tiles_z` the launch's other
+// two dimensions.
 template <int EPI, typename TO>
-static void grouped_mfma_launch(const GroupedArgs& args, int most_rows, int tiles_y, int tiles_z, hipStream_t stream) {
+static void grouped_mfma_launch(const GroupedArgs& args, int most_rows, int tile_rows, int tiles_y, int tiles_z, hipStream_t stream) {
   const int n = args.n;
   if (most_rows <= 64 && args.plan != nullptr) {
     // (only with a plan: its tiles hold at most `most_rows` rows whatever their size; without one, rows come in tiles of the kernel's own size)
@@ -288,10 +307,11 @@ static void grouped_mfma_launch(const GroupedArgs& args, int most_rows, int tile
   const int outputs = EPI == GM_GLU ? 2 * n : n;  // rows of W
   if (outputs <= 128) {
     const int cols = EPI == GM_GLU ? 64 : 128;
-    grouped_mfma_kernel<EPI, TO, 2><<<dim3((n + cols - 1) / cols, tiles_y, tiles_z), 256, 0, stream>>>(args);
+    grouped_mfma_kernel<EPI, TO, 2, 4><<<dim3((n + cols - 1) / cols, tiles_y, tiles_z), 256, 0, stream>>>(args);
   } else {
     const int cols = EPI == GM_GLU ? 128 : 256;
-    grouped_mfma_kernel<EPI, TO, 4><<<dim3((n + cols - 1) / cols, tiles_y, tiles_z), 256, 0, stream>>>(args);
+    if (tile_rows == 128) grouped_mfma_kernel<EPI, TO, 4, 8><<<dim3((n + cols - 1) / cols, tiles_y, tiles_z), 256, 0, stream>>>(args);
+    else grouped_mfma_kernel<EPI, TO, 4, 4><<<dim3((n + cols - 1) / cols, tiles_y, tiles_z), 256, 0, stream>>>(args);
   }
 }
 

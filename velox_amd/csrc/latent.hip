@@ -203,8 +203,8 @@ extern "C" int velox_head_linear(const void* x, int x_width, int x_stride, int x
     args.gate_ld = gate_width;
     const int row_tiles = (m + GM_ROWS - 1) / GM_ROWS;
     if (row_tiles > 65535) return -1;
-    if (gate) grouped_mfma_launch<GM_GATE, bf16_t>(args, m, row_tiles, groups, stream);
-    else grouped_mfma_launch<GM_PLAIN, bf16_t>(args, m, row_tiles, groups, stream);
+    if (gate) grouped_mfma_launch<GM_GATE, bf16_t>(args, m, GM_ROWS, row_tiles, groups, stream);
+    else grouped_mfma_launch<GM_PLAIN, bf16_t>(args, m, GM_ROWS, row_tiles, groups, stream);
     VELOX_RETURN_LAUNCH_STATUS();
   }
   dim3 grid((n + HL_BN - 1) / HL_BN, (m + HL_BM - 1) / HL_BM, groups);

@@ -68,11 +68,13 @@ extern "C" int velox_route_top(const float* logits, int* choice, float* weight, 
 
 // ---------------------------------------------------------------------------------------------
 // The plan, int32: [0] number of tiles, [1 .. 1 + E] first sorted row of every expert and the total, then order[P]
-// (sorted row -> pair = token * top + k), place[P] (pair -> sorted row), tile_expert[max_tiles], tile_row[max_tiles].
+// (sorted row -> pair = token * top + k), place[P] (pair -> sorted row), tile_expert[max_tiles], tile_row[max_tiles]; a tile
+// is up to tile_rows consecutive sorted rows of one expert.
 // ---------------------------------------------------------------------------------------------
 #define PLAN_MAX_EXPERTS 2048
 
-__global__ void __launch_bounds__(1024) routed_plan_kernel(const int* __restrict__ choice, int pairs, int experts, int max_tiles, int* __restrict__ plan) {
+__global__ void __launch_bounds__(1024) routed_plan_kernel(const int* __restrict__ choice, int pairs, int experts, int max_tiles, int tile_rows,
+                                                           int* __restrict__ plan) {
   __shared__ int count[PLAN_MAX_EXPERTS];
   __shared__ int first[PLAN_MAX_EXPERTS + 1];
   int* num_tiles = plan;
@@ -93,7 +95,7 @@ __global__ void __launch_bounds__(1024) routed_plan_kernel(const int* __restrict
     for (int e = 0; e < experts; ++e) {
       first[e] = at;
       starts[e] = at;
-      for (int r = 0; r < count[e] && tiles < max_tiles; r += RT_BM) {
+      for (int r = 0; r < count[e] && tiles < max_tiles; r += tile_rows) {
         tile_expert[tiles] = e;
         tile_row[tiles] = at + r;
         ++tiles;
@@ -122,10 +124,12 @@ extern "C" long long velox_routed_plan_elems(int pairs, int experts) {
 
 extern "C" int velox_routed_max_tiles(int pairs, int experts) { return (pairs + RT_BM - 1) / RT_BM + experts; }
 
-extern "C" int velox_routed_plan(const int* choice, int pairs, int experts, int* plan, hipStream_t stream) {
+// tile_rows: 64, or 128 for the matrix-core products of a step with many rows per expert.  The plan's layout is that of
+// 64-row tiles either way (the most tiles there can be).
+extern "C" int velox_routed_plan(const int* choice, int pairs, int experts, int* plan, int tile_rows, hipStream_t stream) {
   if (pairs <= 0) return 0;
-  if (experts < 1 || experts > PLAN_MAX_EXPERTS) return -1;
-  routed_plan_kernel<<<1, 1024, 0, stream>>>(choice, pairs, experts, velox_routed_max_tiles(pairs, experts), plan);
+  if (experts < 1 || experts > PLAN_MAX_EXPERTS || (tile_rows != RT_BM && tile_rows != 2 * RT_BM)) return -1;
+  routed_plan_kernel<<<1, 1024, 0, stream>>>(choice, pairs, experts, velox_routed_max_tiles(pairs, experts), tile_rows, plan);
   VELOX_RETURN_LAUNCH_STATUS();
 }
 
@@ -315,7 +319,7 @@ static GroupedArgs routed_args(const void* a, const void* w, void* out, const in
 // inter % 8 == 0 (the caller checks).
 extern "C" int velox_routed_products_bf16(const void* x, const void* gate_up, const void* down, void* sorted, void* act, float* y, const int* plan,
                                           const float* pair_weight, int pairs, int experts, int top, int inter, int hidden, int scale_input,
-                                          hipStream_t stream) {
+                                          int tile_rows, hipStream_t stream) {
   if (pairs <= 0) return 0;
   if (hidden % 8 != 0 || inter % 8 != 0) return -1;
   const int max_tiles = velox_routed_max_tiles(pairs, experts);
@@ -323,11 +327,11 @@ extern "C" int velox_routed_products_bf16(const void* x, const void* gate_up, co
   const int* order = plan + 1 + (experts + 1);
   routed_gather_kernel<<<pairs, 256, 0, stream>>>((const bf16_t*)x, order, pair_weight, (bf16_t*)sorted, top, hidden, scale_input);
   GroupedArgs glu = routed_args(sorted, gate_up, act, plan, pairs, experts, inter, hidden, 2 * inter);
-  grouped_mfma_launch<GM_GLU, bf16_t>(glu, pairs, max_tiles, 1, stream);
+  grouped_mfma_launch<GM_GLU, bf16_t>(glu, pairs, tile_rows, max_tiles, 1, stream);
   GroupedArgs last = routed_args(act, down, y, plan, pairs, experts, hidden, inter, hidden);
   last.row_scale = pair_weight;
-  if (scale_input) grouped_mfma_launch<GM_PLAIN, float>(last, pairs, max_tiles, 1, stream);
-  else grouped_mfma_launch<GM_ROW_SCALE, float>(last, pairs, max_tiles, 1, stream);
+  if (scale_input) grouped_mfma_launch<GM_PLAIN, float>(last, pairs, tile_rows, max_tiles, 1, stream);
+  else grouped_mfma_launch<GM_ROW_SCALE, float>(last, pairs, tile_rows, max_tiles, 1, stream);
   VELOX_RETURN_LAUNCH_STATUS();
 }
 
