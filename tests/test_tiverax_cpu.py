@@ -66,7 +66,7 @@ def test_every_tensor_is_named_and_shaped_as_the_design_says(tmp_path):
     assert caught.value.unexpected == ["l1.mix.dkv"] and caught.value.missing == ["l0.mlp.shared.up"]
 
 
-@pytest.mark.parametrize("dims,base,stretch", [(8, 10000.0, (4.0, 24, 8.0, 1.0)), (16, 1e6, (2.0, 1024, 32.0, 1.0)), (12, 500.0, None), (2, 10.0, (8.0, 4, 2.0, 0.5))])
+@pytest.mark.parametrize("dims,base,stretch", [(8, 10000.0, (4.0, 24, 8.0, 1.0)), (24, 2e5, (3.0, 512, 16.0, 2.0)), (12, 500.0, None), (2, 10.0, (8.0, 4, 2.0, 0.5))])
 def test_rotation_tables_hold_the_stretched_frequencies_and_the_magnitude(dims, base, stretch):
     part = make_part("position", "rotary", rotary_dim=dims, theta=base, max_position=300, layout="interleaved", stretch=stretch)
     part.finalize(torch.device("cpu"), torch.float32)

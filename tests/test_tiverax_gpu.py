@@ -67,7 +67,7 @@ def test_embedding_scale_and_two_term_delta(ops, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("heads,dim,rot,rank,half,interleaved,own", [(4, 32, 32, 64, 16, True, True), (3, 12, 16, 40, 6, True, True), (2, 16, 8, 20, 4, False, True),
+@pytest.mark.parametrize("heads,dim,rot,rank,half,interleaved,own", [(6, 48, 16, 96, 8, True, True), (3, 12, 16, 40, 6, True, True), (2, 16, 8, 20, 4, False, True),
                                                                     (5, 8, 6, 9, 3, True, False), (1, 4, 2, 3, 0, True, True)])
 def test_rotation_latent_norm_and_cache_write(ops, dtype, heads, dim, rot, rank, half, interleaved, own):
     ref, dt = TorchOps(), DTYPES[dtype]
@@ -128,7 +128,7 @@ def test_router_scores_and_choices(ops, score, renormalize):
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("tokens,hidden,inter,experts,top,scale_input,with_shared", [(70, 64, 32, 4, 2, True, True), (9, 88, 20, 6, 3, True, False), (300, 96, 40, 8, 1, False, True),
-                                                                                   (1, 320, 96, 8, 1, True, True), (150, 72, 130, 3, 2, False, False),
+                                                                                   (1, 256, 64, 12, 1, True, True), (150, 72, 130, 3, 2, False, False),
                                                                                    (700, 136, 72, 2, 2, True, True), (900, 192, 80, 3, 1, False, False)])
 def test_routed_experts_against_the_plain_loop(ops, dtype, tokens, hidden, inter, experts, top, scale_input, with_shared):
     ref, dt = TorchOps(), DTYPES[dtype]
@@ -176,7 +176,7 @@ def test_routed_experts_part_against_the_design(ops):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("nh,nkv,d,window", [(4, 1, 272, None), (6, 2, 320, None), (2, 2, 1024, 37)])
+@pytest.mark.parametrize("nh,nkv,d,window", [(4, 1, 272, None), (6, 2, 336, None), (2, 2, 1024, 37)])
 def test_attention_for_head_sizes_beyond_the_tiled_kernels(ops, dtype, nh, nkv, d, window):
     """Head sizes above 256 go to the plain kernel: portions behind a context, single tokens and a first token in one step."""
     ref, dt = TorchOps(), DTYPES[dtype]
