@@ -22,47 +22,66 @@
 #define RT_FOLD 128
 
 // ---------------------------------------------------------------------------------------------
-// route_top: one thread per token.  score = sigmoid(z) or softmax(z) over all experts; the `top` largest scores, ties to
-// the lower index; weights are the chosen scores, divided by their sum when `renormalize`.
+// route_top: one wave per token, its lanes over the experts.  score = sigmoid(z) or softmax(z) over all experts; the `top`
+// largest scores, ties to the lower index; weights are the chosen scores, divided by their sum when `renormalize`.
+// Every round the wave takes the largest score that is not yet taken (value first, then the lower index), so the choices
+// come out in descending order of score.
 // ---------------------------------------------------------------------------------------------
-__global__ void __launch_bounds__(128) route_top_kernel(const float* __restrict__ logits, int* __restrict__ choice, float* __restrict__ weight, int tokens,
+#define ROUTE_PER_LANE 32  // experts per lane held in registers: up to 2,048 experts
+
+__global__ void __launch_bounds__(256) route_top_kernel(const float* __restrict__ logits, int* __restrict__ choice, float* __restrict__ weight, int tokens,
                                                         int experts, int top, int softmax, int renormalize) {
-  const int t = blockIdx.x * blockDim.x + threadIdx.x;
-  if (t >= tokens) return;
+  const int lane = threadIdx.x & 63;
+  const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (t >= tokens) return;  // (a whole wave; nothing below crosses waves)
   const float* z = logits + (size_t)t * experts;
   float shift = 0.f, denom = 1.f;
   if (softmax) {
-    shift = z[0];
-    for (int e = 1; e < experts; ++e) shift = fmaxf(shift, z[e]);
-    denom = 0.f;
-    for (int e = 0; e < experts; ++e) denom += expf(z[e] - shift);
+    float m = -INFINITY;
+    for (int e = lane; e < experts; e += 64) m = fmaxf(m, z[e]);
+    shift = wave_max(m);
+    float sum = 0.f;
+    for (int e = lane; e < experts; e += 64) sum += expf(z[e] - shift);
+    denom = wave_sum(sum);
   }
-  int* mine = choice + (size_t)t * top;
-  float* w = weight + (size_t)t * top;
-  float sum = 0.f;
+  float score[ROUTE_PER_LANE];
+#pragma unroll
+  for (int u = 0; u < ROUTE_PER_LANE; ++u) {
+    const int e = lane + 64 * u;
+    score[u] = -1.f;  // (scores are positive: -1 marks "no such expert" and "taken")
+    if (e < experts) score[u] = softmax ? expf(z[e] - shift) / denom : 1.f / (1.f + expf(-z[e]));
+  }
+  float total = 0.f;
   for (int k = 0; k < top; ++k) {
-    int best = -1;
-    float best_score = 0.f;
-    for (int e = 0; e < experts; ++e) {
-      bool taken = false;
-      for (int j = 0; j < k; ++j) taken |= mine[j] == e;
-      if (taken) continue;
-      const float s = softmax ? expf(z[e] - shift) / denom : 1.f / (1.f + expf(-z[e]));
-      if (best < 0 || s > best_score) { best = e; best_score = s; }
+    float best = -1.f;
+    int best_e = 0x7fffffff;
+#pragma unroll
+    for (int u = 0; u < ROUTE_PER_LANE; ++u)
+      if (score[u] > best) { best = score[u]; best_e = lane + 64 * u; }  // (ascending e within a lane: the first of equals stays)
+#pragma unroll
+    for (int offset = 32; offset > 0; offset >>= 1) {
+      const float other = __shfl_xor(best, offset, 64);
+      const int other_e = __shfl_xor(best_e, offset, 64);
+      if (other > best || (other == best && other_e < best_e)) { best = other; best_e = other_e; }
     }
-    mine[k] = best;
-    w[k] = best_score;
-    sum += best_score;
+#pragma unroll
+    for (int u = 0; u < ROUTE_PER_LANE; ++u)
+      if (lane + 64 * u == best_e) score[u] = -1.f;
+    total += best;
+    if (lane == 0) {
+      choice[(size_t)t * top + k] = best_e;
+      weight[(size_t)t * top + k] = best;
+    }
   }
-  if (renormalize)
-    for (int k = 0; k < top; ++k) w[k] /= sum;
+  if (renormalize && lane == 0)  // (the lane that wrote them)
+    for (int k = 0; k < top; ++k) weight[(size_t)t * top + k] /= total;
 }
 
 extern "C" int velox_route_top(const float* logits, int* choice, float* weight, int tokens, int experts, int top, int softmax, int renormalize,
                                hipStream_t stream) {
   if (tokens <= 0) return 0;
-  if (experts < 1 || top < 1 || top > experts) return -1;
-  route_top_kernel<<<(tokens + 127) / 128, 128, 0, stream>>>(logits, choice, weight, tokens, experts, top, softmax, renormalize);
+  if (experts < 1 || experts > 64 * ROUTE_PER_LANE || top < 1 || top > experts) return -1;
+  route_top_kernel<<<(tokens + 3) / 4, 256, 0, stream>>>(logits, choice, weight, tokens, experts, top, softmax, renormalize);
   VELOX_RETURN_LAUNCH_STATUS();
 }
 
@@ -72,11 +91,16 @@ extern "C" int velox_route_top(const float* logits, int* choice, float* weight, 
 // is up to tile_rows consecutive sorted rows of one expert.
 // ---------------------------------------------------------------------------------------------
 #define PLAN_MAX_EXPERTS 2048
+#define PLAN_COPY_PAIRS 64  // up to this many pairs the plan kernel can copy the rows itself
 
+// With `sorted` the kernel also copies the rows of x into the plan's order (scaled by the pair's weight when `scale`), what
+// routed_gather_kernel does: for steps of few pairs, which then run one kernel less.
 __global__ void __launch_bounds__(1024) routed_plan_kernel(const int* __restrict__ choice, int pairs, int experts, int max_tiles, int tile_rows,
-                                                           int* __restrict__ plan) {
+                                                           int* __restrict__ plan, const bf16_t* __restrict__ x, bf16_t* __restrict__ sorted,
+                                                           const float* __restrict__ pair_weight, int top, int hidden, int scale) {
   __shared__ int count[PLAN_MAX_EXPERTS];
   __shared__ int first[PLAN_MAX_EXPERTS + 1];
+  __shared__ int order_s[PLAN_COPY_PAIRS];
   int* num_tiles = plan;
   int* starts = plan + 1;
   int* order = starts + experts + 1;
@@ -114,6 +138,23 @@ __global__ void __launch_bounds__(1024) routed_plan_kernel(const int* __restrict
     const int row = first[e] + atomicAdd(&count[e], 1);
     order[row] = p;
     place[p] = row;
+    if (sorted != nullptr) order_s[row] = p;
+  }
+  if (sorted == nullptr) return;  // (uniform over the workgroup)
+  __syncthreads();
+  // the rows of x in the plan's order, 16 bytes per thread at a time (the caller checked hidden % 8 == 0 and pairs <= PLAN_COPY_PAIRS)
+  const int pieces = hidden / 8;
+  for (int at = threadIdx.x; at < first[experts] * pieces; at += blockDim.x) {  // (first[experts]: the pairs that were placed)
+    const int row = at / pieces, piece_at = at % pieces;
+    const int p = order_s[row];
+    float4_t piece = reinterpret_cast<const float4_t*>(x + (size_t)(p / top) * hidden)[piece_at];
+    if (scale) {
+      const float w = pair_weight[p];
+      bf16_t* e8 = reinterpret_cast<bf16_t*>(&piece);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) e8[j] = from_f32<bf16_t>(to_f32(e8[j]) * w);
+    }
+    reinterpret_cast<float4_t*>(sorted + (size_t)row * hidden)[piece_at] = piece;
   }
 }
 
@@ -126,10 +167,14 @@ extern "C" int velox_routed_max_tiles(int pairs, int experts) { return (pairs + 
 
 // tile_rows: 64, or 128 for the matrix-core products of a step with many rows per expert.  The plan's layout is that of
 // 64-row tiles either way (the most tiles there can be).
-extern "C" int velox_routed_plan(const int* choice, int pairs, int experts, int* plan, int tile_rows, hipStream_t stream) {
+// x, sorted, pair_weight, top, hidden, scale: see routed_plan_kernel (sorted == nullptr: the plan alone).
+extern "C" int velox_routed_plan(const int* choice, int pairs, int experts, int* plan, int tile_rows, const void* x, void* sorted, const float* pair_weight,
+                                 int top, int hidden, int scale, hipStream_t stream) {
   if (pairs <= 0) return 0;
   if (experts < 1 || experts > PLAN_MAX_EXPERTS || (tile_rows != RT_BM && tile_rows != 2 * RT_BM)) return -1;
-  routed_plan_kernel<<<1, 1024, 0, stream>>>(choice, pairs, experts, velox_routed_max_tiles(pairs, experts), tile_rows, plan);
+  if (sorted != nullptr && (x == nullptr || pairs > PLAN_COPY_PAIRS || hidden % 8 != 0 || top < 1 || (((uintptr_t)x | (uintptr_t)sorted) & 15) != 0)) return -1;
+  routed_plan_kernel<<<1, 1024, 0, stream>>>(choice, pairs, experts, velox_routed_max_tiles(pairs, experts), tile_rows, plan, (const bf16_t*)x, (bf16_t*)sorted,
+                                             pair_weight, top, hidden, scale);
   VELOX_RETURN_LAUNCH_STATUS();
 }
 
@@ -325,7 +370,8 @@ extern "C" int velox_routed_products_bf16(const void* x, const void* gate_up, co
   const int max_tiles = velox_routed_max_tiles(pairs, experts);
   if (max_tiles > 65535) return -1;
   const int* order = plan + 1 + (experts + 1);
-  routed_gather_kernel<<<pairs, 256, 0, stream>>>((const bf16_t*)x, order, pair_weight, (bf16_t*)sorted, top, hidden, scale_input);
+  if (x != nullptr)  // (nullptr: the plan kernel has copied the rows already)
+    routed_gather_kernel<<<pairs, 256, 0, stream>>>((const bf16_t*)x, order, pair_weight, (bf16_t*)sorted, top, hidden, scale_input);
   GroupedArgs glu = routed_args(sorted, gate_up, act, plan, pairs, experts, inter, hidden, 2 * inter);
   grouped_mfma_launch<GM_GLU, bf16_t>(glu, pairs, tile_rows, max_tiles, 1, stream);
   GroupedArgs last = routed_args(act, down, y, plan, pairs, experts, hidden, inter, hidden);
@@ -341,11 +387,18 @@ extern "C" int velox_routed_products_bf16(const void* x, const void* gate_up, co
 template <typename T>
 __global__ void __launch_bounds__(256) routed_combine_kernel(const float* __restrict__ y, const int* __restrict__ place, const T* __restrict__ shared,
                                                              T* __restrict__ out, int top, int hidden) {
+  __shared__ int rows[64];  // the token's rows of y, looked up once (up to 64 choices; more are looked up as they are added)
   const int t = blockIdx.x;
+  const int* mine = place + (size_t)t * top;
+  if (top <= 64) {
+    if (threadIdx.x < top) rows[threadIdx.x] = mine[threadIdx.x];
+    __syncthreads();
+    mine = rows;
+  }
   for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
     float v = 0.f;
     for (int k = 0; k < top; ++k) {
-      const int row = place[(size_t)t * top + k];
+      const int row = mine[k];
       if (row >= 0) v += y[(size_t)row * hidden + i];
     }
     if (shared) v += to_f32(shared[(size_t)t * hidden + i]);

@@ -63,9 +63,25 @@ def build_dirs() -> List[str]:
     return dirs
 
 
+def _headers_of(sources: Sequence[str]) -> List[str]:
+    """The headers of this folder that the sources include, directly or through one another, in a fixed order."""
+    found: List[str] = []
+    todo = list(sources)
+    while todo:
+        with open(os.path.join(SOURCE_DIR, todo.pop(0)), "r", encoding="utf-8") as handle:
+            for line in handle:
+                line = line.strip()
+                if line.startswith('#include "'):
+                    name = line.split('"')[1]
+                    if name in HEADERS and name not in found:
+                        found.append(name)
+                        todo.append(name)
+    return sorted(found)
+
+
 def _digest(sources: Sequence[str], defines: Dict[str, object]) -> str:
     h = hashlib.sha1()
-    for name in list(sources) + HEADERS:
+    for name in list(sources) + _headers_of(sources):  # (a header that a library does not include does not make it stale)
         with open(os.path.join(SOURCE_DIR, name), "rb") as handle:
             h.update(name.encode())
             h.update(handle.read())

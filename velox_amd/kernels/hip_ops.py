@@ -79,6 +79,7 @@ def _weight_of(weight) -> Tuple[torch.Tensor, Optional[PreparedWeight]]:
 class HipOps:
     name = "hip-gfx950"
     MAX_TILED_HEAD_DIM = 256  # head sizes above this go to the plain attention kernel
+    FEW_PAIRS = 64  # up to this many (token, expert) pairs the experts' plan kernel copies the rows itself
 
     def __init__(self, device) -> None:
         self.device = torch.device(device)
@@ -146,7 +147,7 @@ class HipOps:
         c.velox_route_top.argtypes = [_P, _P, _P, _I, _I, _I, _I, _I, _P]
         c.velox_routed_plan_elems.argtypes = [_I, _I]
         c.velox_routed_plan_elems.restype = ctypes.c_longlong
-        c.velox_routed_plan.argtypes = [_P, _I, _I, _P, _I, _P]
+        c.velox_routed_plan.argtypes = [_P, _I, _I, _P, _I, _P, _P, _P, _I, _I, _I, _P]
         c.velox_grouped_glu.argtypes = [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P]
         c.velox_grouped_down.argtypes = [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P]
         c.velox_routed_combine.argtypes = [_P, _P, _P, _P, _I, _I, _I, _I, _I, _P]
@@ -853,13 +854,17 @@ class HipOps:
         on_matrix_cores = x.dtype == torch.bfloat16 and hidden % 8 == 0 and inter % 8 == 0 and self.use_grouped_mfma
         # tiles of 128 rows for the matrix cores when the experts have that many rows on average (W is then read half as often)
         tile_rows = 128 if on_matrix_cores and pairs >= 128 * num_experts and 2 * inter > 128 and hidden > 128 else 64
-        self._launched(self._core.velox_routed_plan(_ptr(choice), pairs, num_experts, _ptr(plan), tile_rows, self._stream()), "routed_plan")
+        # few pairs: the plan's kernel also copies the rows into its order, and the step runs one kernel less
+        ordered = torch.empty((pairs, hidden), dtype=x.dtype, device=self.device) if on_matrix_cores else None
+        copied_by_plan = on_matrix_cores and pairs <= self.FEW_PAIRS
+        self._launched(self._core.velox_routed_plan(_ptr(choice), pairs, num_experts, _ptr(plan), tile_rows, _ptr(x) if copied_by_plan else _P(0),
+                                                    _ptr(ordered) if copied_by_plan else _P(0), _ptr(weight), top, hidden, int(bool(scale_input)), self._stream()),
+                       "routed_plan")
         act = torch.empty((pairs, inter), dtype=x.dtype, device=self.device)
         y = torch.empty((pairs, hidden), dtype=torch.float32, device=self.device)
         if on_matrix_cores:
             # bfloat16 rows of whole 16-byte pieces: sorted copies of the rows, then both products on the matrix cores
-            ordered = torch.empty((pairs, hidden), dtype=x.dtype, device=self.device)
-            self._launched(self._core.velox_routed_products_bf16(_ptr(x), _ptr(gate_up_weight), _ptr(down_weight), _ptr(ordered), _ptr(act), _ptr(y), _ptr(plan),
+            self._launched(self._core.velox_routed_products_bf16(_P(0) if copied_by_plan else _ptr(x), _ptr(gate_up_weight), _ptr(down_weight), _ptr(ordered), _ptr(act), _ptr(y), _ptr(plan),
                                                                  _ptr(weight), pairs, num_experts, top, inter, hidden, int(bool(scale_input)), tile_rows,
                                                                  self._stream()), "routed_products")
             return self._routed_combine(y, plan, shared, tokens, top, num_experts, hidden, out_dtype)
