@@ -102,6 +102,62 @@ class TorchOps:
         var = (x * x).sum(-1, keepdim=True) / x.shape[-1]
         return (x * torch.rsqrt(var + eps) * weight.float()).to(out_dtype)
 
+    def add_sinusoid(self, hidden, positions, frequencies):
+        """hidden[t, 2i] += sin(p_t f_i), hidden[t, 2i + 1] += cos(p_t f_i), in place."""
+        angle = positions.double()[:, None] * frequencies.double()[None, :]
+        width = hidden.shape[1]
+        hidden[:, 0::2] += torch.sin(angle).float()[:, : (width + 1) // 2]
+        hidden[:, 1::2] += torch.cos(angle).float()[:, : width // 2]
+        return hidden
+
+    def add_cast(self, residual, delta, out_dtype):
+        if delta is not None:
+            residual += delta.float()
+        return residual if out_dtype == torch.float32 else residual.to(out_dtype)
+
+    def norm_add(self, residual, delta, weight, eps, mult, out_dtype):
+        y = delta.float().sum(0) if delta.dim() == 3 else delta.float()
+        var = (y * y).sum(-1, keepdim=True) / y.shape[-1]
+        residual += mult * (y / torch.sqrt(var + eps) * weight.float())
+        return residual if out_dtype == torch.float32 else residual.to(out_dtype)
+
+    def qk_norm_write(self, qkv, num_heads, num_kv_heads, dim, vdim, cached_dim, q_norm, k_norm, whole, eps, q_temp, positions, first_values,
+                      mix_weight, slot_mapping, k_cache, v_cache, block_size, write_kv=True):
+        t = qkv.shape[0]
+        q_size, k_size, v_size = num_heads * dim, num_kv_heads * dim, num_kv_heads * vdim
+        wide = qkv.float()
+        q, k, v = wide[:, :q_size], wide[:, q_size:q_size + k_size], wide[:, q_size + k_size:q_size + k_size + v_size]
+
+        def unit(x):
+            return x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps)
+
+        if whole:
+            q = (unit(q) * q_norm.float()).view(t, num_heads, dim)
+            k = (unit(k) * k_norm.float()).view(t, num_kv_heads, dim)
+        else:
+            q = unit(q.reshape(t, num_heads, dim)) * q_norm.float()
+            k = unit(k.reshape(t, num_kv_heads, dim)) * k_norm.float()
+        if q_temp is not None:
+            coef, every = q_temp
+            steps = torch.div(positions.long() + 1, int(every), rounding_mode="floor") + 1
+            q = q * (1.0 + coef * torch.log(steps.float()))[:, None, None]
+        if first_values is not None:
+            source, offset = first_values
+            lam = mix_weight.float().reshape(())
+            v = (1.0 - lam) * v + lam * source[:, offset:offset + v_size].float()
+        out = torch.zeros((t, num_heads, cached_dim), dtype=qkv.dtype, device=qkv.device)
+        out[:, :, :dim] = q.to(qkv.dtype)
+        if write_kv:
+            pages = slot_mapping.long() // block_size
+            offsets = slot_mapping.long() % block_size
+            keys = torch.zeros((t, num_kv_heads, cached_dim), dtype=k_cache.dtype, device=qkv.device)
+            keys[:, :, :dim] = k.to(k_cache.dtype)
+            values = torch.zeros((t, num_kv_heads, cached_dim), dtype=v_cache.dtype, device=qkv.device)
+            values[:, :, :vdim] = v.reshape(t, num_kv_heads, vdim).to(v_cache.dtype)
+            k_cache[pages, :, offsets, :] = keys
+            v_cache[pages, :, :, offsets] = values
+        return out.view(t, num_heads * cached_dim)
+
     # -- matrix products ----------------------------------------------------------------
     def linear(self, x, weight, bias, out_dtype, partials_ok=False, residual_norm=None):
         out = x.float() @ weight.float().T
@@ -202,20 +258,29 @@ class TorchOps:
         return out
 
     # -- routed experts -------------------------------------------------------------------
-    def route_top(self, logits, top, score="sigmoid", renormalize=False):
+    def route_top(self, logits, top, score="sigmoid", renormalize=False, correction=None):
         scores = torch.sigmoid(logits.float()) if score == "sigmoid" else torch.softmax(logits.float(), dim=-1)
-        weight, choice = scores.topk(top, dim=-1)
+        if correction is not None:  # the correction steers the choice only
+            choice = (scores + correction.float()).topk(top, dim=-1).indices
+            weight = scores.gather(-1, choice)
+        else:
+            weight, choice = scores.topk(top, dim=-1)
         if renormalize:
             weight = weight / weight.sum(-1, keepdim=True)
         return choice.to(torch.int32), weight
 
-    def routed_experts(self, x, choice, weight, gate_up_weight, down_weight, num_experts, scale_input, shared, out_dtype, workspace=None):
+    def routed_experts(self, x, choice, weight, gate_up_weight, down_weight, num_experts, scale_input, shared, out_dtype, workspace=None,
+                       unit=(1.0, float("inf"), 0.0), identity_experts=0):
+        alpha, limit, shift = unit
         t, h = x.shape
         f = gate_up_weight.shape[0] // (2 * num_experts)
         gate_up = gate_up_weight.view(num_experts, 2 * f, h).float()
         down = down_weight.view(num_experts, h, f).float()
         out = torch.zeros((t, h), dtype=torch.float32, device=x.device)
         for k in range(choice.shape[1]):  # a token's results are added in the order of its choices
+            rows = (choice[:, k] >= num_experts).nonzero().flatten()
+            if rows.numel():  # identity experts: the input itself, times the weight
+                out[rows] += x[rows].float() * weight[rows, k:k + 1]
             for e in range(num_experts):
                 rows = (choice[:, k] == e).nonzero().flatten()
                 if not rows.numel():
@@ -223,7 +288,8 @@ class TorchOps:
                 w = weight[rows, k:k + 1]
                 a = (x[rows].float() * w).to(x.dtype).float() if scale_input else x[rows].float()
                 both = a @ gate_up[e].T
-                act = (both[:, :f] * torch.sigmoid(both[:, :f]) * both[:, f:]).to(x.dtype).float()
+                gate, up = both[:, :f].clamp(max=limit), both[:, f:].clamp(min=-limit, max=limit)
+                act = (gate * torch.sigmoid(alpha * gate) * (up + shift)).to(x.dtype).float()
                 y = act @ down[e].T
                 out[rows] += y if scale_input else y * w
         if shared is not None:
@@ -231,7 +297,9 @@ class TorchOps:
         return out.to(out_dtype)
 
     # -- attention over the paged cache -------------------------------------------------
-    def paged_attention(self, qkv, num_heads, num_kv_heads, head_dim, k_cache, v_cache, block_size, block_tables, cu_q, kv_lens, max_q_len, max_kv_len, scale, window, all_decode, workspace, splits=None, decode_prefix=0, portions_max_kv_len=None):
+    def paged_attention(self, qkv, num_heads, num_kv_heads, head_dim, k_cache, v_cache, block_size, block_tables, cu_q, kv_lens, max_q_len, max_kv_len, scale, window, all_decode, workspace, splits=None, decode_prefix=0, portions_max_kv_len=None,
+                        distance_bias=None):
+        """``distance_bias``: float32 [heads, L]; the score of a key ``n`` behind the query gets column ``min(n, L - 1)``."""
         t = qkv.shape[0]
         group = num_heads // num_kv_heads
         q_all = qkv[:, : num_heads * head_dim].view(t, num_heads, head_dim)
@@ -254,6 +322,9 @@ class TorchOps:
             for h in range(num_heads):
                 kv = h // group
                 scores = (q_all[lo:hi, h].float() @ keys[:, kv].T) * scale
+                if distance_bias is not None:
+                    behind = (q_pos[:, None] - index[None, :]).clamp(min=0, max=distance_bias.shape[1] - 1)
+                    scores = scores + distance_bias[h].float()[behind]
                 scores = scores.masked_fill(~keep, float("-inf"))
                 m = scores.max(-1, keepdim=True).values
                 p = torch.exp(scores - m)

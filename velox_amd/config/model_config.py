@@ -28,6 +28,31 @@ def read_config_json(model_dir: str) -> Dict[str, Any]:
     return raw
 
 
+def read_tensor_shapes(model_dir: str) -> Dict[str, List[int]]:
+    """name -> shape of every tensor in the folder's safetensors files, from their headers alone (8 bytes of length, then
+    that many bytes of JSON); for architectures in which a size is given by a tensor's shape and not by ``config.json``."""
+    import struct
+
+    index = os.path.join(model_dir, "model.safetensors.index.json")
+    if os.path.isfile(index):
+        with open(index, "r", encoding="utf-8") as handle:
+            files = sorted(set(json.load(handle)["weight_map"].values()))
+    else:
+        files = ["model.safetensors"]
+    shapes: Dict[str, List[int]] = {}
+    for name in files:
+        path = os.path.join(model_dir, name)
+        if not os.path.isfile(path):
+            raise ConfigError(f"{model_dir!r} holds no {name}")
+        with open(path, "rb") as handle:
+            (length,) = struct.unpack("<Q", handle.read(8))
+            header = json.loads(handle.read(length).decode("utf-8"))
+        for tensor, entry in header.items():
+            if tensor != "__metadata__":
+                shapes[tensor] = [int(n) for n in entry["shape"]]
+    return shapes
+
+
 def require(raw: Dict[str, Any], key: str, kind):
     if key not in raw or raw[key] is None:
         raise ConfigError(f"config.json is missing required key {key!r}")

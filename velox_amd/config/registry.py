@@ -9,7 +9,7 @@ from __future__ import annotations
 from dataclasses import dataclass
 from typing import Any, Callable, Dict
 
-from .model_config import ConfigError, ModelConfig, read_config_json
+from .model_config import ConfigError, ModelConfig, read_config_json, read_tensor_shapes
 
 
 @dataclass(frozen=True)
@@ -17,16 +17,19 @@ class Architecture:
     name: str
     read_config: Callable[[Dict[str, Any]], ModelConfig]
     make_spec: Callable[..., Any]  # (config, max_position) -> ModelSpec
+    reads_tensor_shapes: bool = False
 
 
 _ARCHITECTURES: Dict[str, Architecture] = {}
 _ARCHITECTURE_OF_MODEL_TYPE: Dict[str, str] = {}
 
 
-def register_architecture(name: str, read_config, make_spec, model_types=()) -> None:
+def register_architecture(name: str, read_config, make_spec, model_types=(), reads_tensor_shapes: bool = False) -> None:
     """``name`` is what ``config.json`` holds in ``architectures[0]``; ``model_types`` are values of its ``model_type``
-    key that stand for this class when ``architectures`` is left out."""
-    _ARCHITECTURES[name] = Architecture(name, read_config, make_spec)
+    key that stand for this class when ``architectures`` is left out.  ``reads_tensor_shapes``: some size of this class
+    is given by a tensor's shape only; a folder's configuration then reaches ``read_config`` with the shapes of the
+    folder's tensors under the key ``tensor_shapes``."""
+    _ARCHITECTURES[name] = Architecture(name, read_config, make_spec, bool(reads_tensor_shapes))
     for model_type in model_types:
         _ARCHITECTURE_OF_MODEL_TYPE[model_type] = name
 
@@ -60,7 +63,10 @@ def config_from_dict(raw: Dict[str, Any]) -> ModelConfig:
 
 
 def load_config(model_dir: str) -> ModelConfig:
-    return config_from_dict(read_config_json(model_dir))
+    raw = read_config_json(model_dir)
+    if get_architecture(architecture_name(raw)).reads_tensor_shapes:
+        raw = dict(raw, tensor_shapes=read_tensor_shapes(model_dir))
+    return config_from_dict(raw)
 
 
 def _load_builtin() -> None:

@@ -107,6 +107,9 @@ class StepContext:
     workspace: Workspace
     cache: CacheManager = field(repr=False, default=None)
     decode_prefix: int = 0  # how many of the first sequences bring exactly one token
+    # what a part of an earlier schedule entry leaves for later ones within the step (values that later layers blend
+    # with their own, say): name -> tensor of this step's rows.  Whoever publishes a name writes it anew in every forward.
+    shared: Dict[str, object] = field(default_factory=dict)
 
     def cache_view(self, entry: int):
         return self.cache.view(entry, self.groups)

@@ -1,2 +1,2 @@
 """Architectures built in; importing the package registers them."""
-from . import qwen2, tiverax  # noqa: F401
+from . import dipisun, qwen2, tiverax  # noqa: F401

@@ -3,7 +3,7 @@ from .base import (  # noqa: F401
     PAGE, Block, Embedding, FeedForward, Mixer, Norm, OutputHead, PagedNeed, Param, Part, PartSpec, PositionEncoding, StateNeed,
     fused_rows, make_part, register_arrangement, register_part, single,
 )
-from . import attention, feed_forward, latent_attention, norms, position  # noqa: F401  (register kinds)
+from . import attention, feed_forward, latent_attention, normed_attention, norms, position  # noqa: F401  (register kinds)
 from .attention import kv_pages  # noqa: F401
-from .block import ParallelBlock, PreNormBlock  # noqa: F401
+from .block import OutputNormBlock, ParallelBlock, PreNormBlock  # noqa: F401
 from .model import DecoderModel, LayerSpec, ModelSpec, ScheduleEntry  # noqa: F401

@@ -223,6 +223,15 @@ class DeferredNorm:
         return self.x.dtype
 
 
+@dataclass
+class ResidualCopy:
+    """What a block hands on when it has added everything to the residual itself and holds the updated residual in the
+    run dtype already (``copy``, [T, H]; in a float32 run the residual itself): a norm that gets it as its delta adds
+    nothing, and a block that reads the residual stream directly takes ``copy`` as its input without rounding again."""
+
+    copy: torch.Tensor
+
+
 class Mixer(Part):
     def cache_need(self):
         """``PagedNeed``, ``StateNeed`` or None."""
@@ -260,6 +269,12 @@ class Norm(Part):
         [R]): nothing is changed and ``normalise(residual[rows] + delta[rows])`` comes back.
         """
         raise NotImplementedError
+
+    def add_normed(self, residual: torch.Tensor, delta: torch.Tensor, mult: float, ctx) -> torch.Tensor:
+        """The norm on a sub-layer's OUTPUT: ``residual += mult * normalise(delta)`` in place, in float32 (``delta`` is
+        [T, H] or float32 partial sums [S, T, H]); the updated residual comes back in the run dtype, [T, H] (the
+        residual itself in a float32 run), for the sub-layer that reads it next."""
+        raise NotImplementedError(f"{type(self).__name__} cannot norm a sub-layer's output")
 
 
 class PositionEncoding(Part):

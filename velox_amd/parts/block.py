@@ -5,6 +5,10 @@
 tensor; what a sub-layer produced is carried as ``pending`` and added inside the next
 norm's kernel, so each block hands its feed-forward output on to whoever normalises next.
 
+``OutputNormBlock`` (not in the reference): ``h = h + m * norm1(mixer(h)); h = h + m * norm2(ff(h))``.  The sub-layers
+read the residual stream itself and only their outputs are normed, so nothing is pending between blocks; what is handed
+on is the updated residual in the run dtype (``ResidualCopy``), which the norm's kernel writes beside the float32 sum.
+
 ``ParallelBlock`` (not in the reference): ``n = norm(h); h = h + (mixer(n) + ff(n))``, one norm that both
 sub-layers read.  It hands both outputs on as a ``SumOf``, which the next norm's kernel adds up in float32.
 """
@@ -14,7 +18,7 @@ from typing import Optional, Tuple
 
 import torch
 
-from .base import Block, FeedForward, Mixer, Norm, Part, ResidualSink, SumOf, register_arrangement
+from .base import Block, FeedForward, Mixer, Norm, Part, ResidualCopy, ResidualSink, SumOf, register_arrangement
 
 
 class PreNormBlock(Block):
@@ -80,3 +84,46 @@ class ParallelBlock(Block):
 
 
 register_arrangement("parallel", ParallelBlock)
+
+
+class OutputNormBlock(Block):
+    def __init__(self, prefix: str, mixer: Mixer, feed_forward: FeedForward, mixer_norm: Norm, ff_norm: Norm, residual_mult: float = 1.0) -> None:
+        """``residual_mult``: the factor ``m`` on both normed sub-layer outputs."""
+        super().__init__(prefix)
+        self.mixer = mixer
+        self.feed_forward = feed_forward
+        self.mixer_norm = mixer_norm
+        self.ff_norm = ff_norm
+        self.residual_mult = float(residual_mult)
+        self.has_feed_forward = type(feed_forward).__name__ != "NoFeedForward"
+
+    def children(self) -> Tuple[Part, ...]:
+        if not self.has_feed_forward:
+            return (self.mixer_norm, self.mixer)  # (no second norm: its tensor does not exist)
+        return (self.mixer_norm, self.mixer, self.ff_norm, self.feed_forward)
+
+    def input_norm(self) -> Optional[Norm]:
+        return None  # (the block begins with its mixer)
+
+    @staticmethod
+    def _input(residual: torch.Tensor, pending, ctx) -> torch.Tensor:
+        if isinstance(pending, ResidualCopy):
+            return pending.copy
+        if isinstance(pending, SumOf):
+            first = pending.first.float().sum(0) if pending.first.dim() == 3 else pending.first.float()
+            pending = first + pending.second.float()
+        elif pending is not None and pending.dim() == 3:
+            pending = pending.sum(0)
+        return ctx.ops.add_cast(residual, pending, ctx.dtype)
+
+    def forward(self, residual: torch.Tensor, pending, ctx, cache, owns_cache: bool, next_norm: Optional[Norm] = None):
+        x = self._input(residual, pending, ctx)
+        mixed = self.mixer.forward(x, ctx, cache, owns_cache)
+        x = self.mixer_norm.add_normed(residual, mixed, self.residual_mult, ctx)
+        if self.has_feed_forward:
+            out = self.feed_forward.forward(x, ctx)
+            x = self.ff_norm.add_normed(residual, out, self.residual_mult, ctx)
+        return ResidualCopy(x)
+
+
+register_arrangement("output_norm", OutputNormBlock)

@@ -22,6 +22,9 @@ import torch
 from .base import FeedForward, Param, fused_rows, register_part, single
 
 
+SILU_UNIT = (1.0, float("inf"), 0.0)  # (alpha, limit, shift) of ``silu(gate) * up``
+
+
 class GatedMLP(FeedForward):
     def __init__(self, prefix: str, hidden_size: int, intermediate_size: int, activation: str = "silu",
                  names: Tuple[str, str, str] = ("gate_proj.weight", "up_proj.weight", "down_proj.weight")) -> None:
@@ -85,12 +88,26 @@ class RoutedExperts(FeedForward):
                  renormalize: bool = False, scale_input: bool = True, shared_intermediate_size: Optional[int] = None,
                  expert_names: Tuple[str, str, str] = ("experts.{e}.gate.weight", "experts.{e}.up.weight", "experts.{e}.down.weight"),
                  router_name: str = "router.weight", shared_prefix: str = "shared.",
-                 shared_names: Tuple[str, str, str] = ("gate_proj.weight", "up_proj.weight", "down_proj.weight")) -> None:
+                 shared_names: Tuple[str, str, str] = ("gate_proj.weight", "up_proj.weight", "down_proj.weight"),
+                 unit: Tuple[float, float, float] = SILU_UNIT, identity_experts: int = 0, correction_name: Optional[str] = None) -> None:
+        """``unit = (alpha, limit, shift)``: a unit's middle is ``g sigmoid(alpha g) (u + shift)`` with ``g = min(W_gate x,
+        limit)`` and ``u = clamp(W_up x, -limit, limit)``; ``(1, inf, 0)`` is ``silu(gate) * up``.  ``identity_experts``: the
+        router has that many outputs more than there are units; an identity expert's result is its input (times the
+        weight, wherever the weight stands).  ``correction_name``: a float32 vector over all router outputs that is added
+        to the scores for the choice only; the weights are the scores without it."""
         super().__init__(prefix)
+        self.unit = (float(unit[0]), float(unit[1]), float(unit[2]))
+        if not self.unit[1] > 0:
+            raise ValueError(f"unit: the limit must be positive (inf for none), got {self.unit[1]}")
+        self.identity_experts = int(identity_experts)
+        if self.identity_experts < 0:
+            raise ValueError("identity_experts must not be negative")
+        self.correction_name = correction_name
+        self.correction: Optional[torch.Tensor] = None
         if score not in ("sigmoid", "softmax"):
             raise ValueError(f"score {score!r} is not implemented ('sigmoid' or 'softmax')")
-        if not 1 <= int(top) <= int(num_experts):
-            raise ValueError(f"top={top} must lie between 1 and the number of experts ({num_experts})")
+        if not 1 <= int(top) <= int(num_experts) + int(identity_experts):
+            raise ValueError(f"top={top} must lie between 1 and the number of experts ({int(num_experts) + int(identity_experts)})")
         self.hidden_size = int(hidden_size)
         self.intermediate_size = int(intermediate_size)
         self.num_experts = int(num_experts)
@@ -111,11 +128,14 @@ class RoutedExperts(FeedForward):
         h, f, e = self.hidden_size, self.intermediate_size, self.num_experts
         gate, up, down = self.expert_names
         gate_up_names = tuple(name.format(e=i) for i in range(e) for name in (gate, up))
-        return {
-            "router_weight": single(self.router_name, (e, h)),
+        out = {
+            "router_weight": single(self.router_name, (e + self.identity_experts, h)),
             "gate_up_weight": fused_rows(gate_up_names, ((f, h),) * (2 * e)),
             "down_weight": fused_rows(tuple(down.format(e=i) for i in range(e)), ((h, f),) * e),
         }
+        if self.correction_name is not None:
+            out["correction"] = single(self.correction_name, (e + self.identity_experts,), role="vector")
+        return out
 
     def children(self):
         return (self.shared,) if self.shared is not None else ()
@@ -130,10 +150,16 @@ class RoutedExperts(FeedForward):
         ops = ctx.ops
         x = ops.materialize(x)
         logits = ops.linear(x, self.router_weight, None, torch.float32)
-        choice, weight = ops.route_top(logits, self.top, self.score, self.renormalize)
+        if self.correction is not None:
+            choice, weight = ops.route_top(logits, self.top, self.score, self.renormalize, correction=self.correction)
+        else:
+            choice, weight = ops.route_top(logits, self.top, self.score, self.renormalize)
         shared = self.shared.forward(x, ctx, partials_ok=False) if self.shared is not None else None
+        if self.unit == SILU_UNIT and not self.identity_experts:
+            return ops.routed_experts(x, choice, weight, self.gate_up_weight, self.down_weight, self.num_experts, self.scale_input, shared,
+                                      ctx.dtype, ctx.workspace)
         return ops.routed_experts(x, choice, weight, self.gate_up_weight, self.down_weight, self.num_experts, self.scale_input, shared,
-                                  ctx.dtype, ctx.workspace)
+                                  ctx.dtype, ctx.workspace, unit=self.unit, identity_experts=self.identity_experts)
 
 
 register_part("feed_forward", "routed_experts", RoutedExperts)

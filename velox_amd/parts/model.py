@@ -32,6 +32,7 @@ class LayerSpec:
     ff_norm: PartSpec
     position: Optional[str] = None  # key into ModelSpec.positions handed to the mixer
     arrangement: str = "pre_norm"
+    arrangement_args: Tuple[Tuple[str, object], ...] = ()  # constants of the arrangement (sorted pairs, as in PartSpec)
     # where each part's tensors stand in the checkpoint, below the layer's prefix (an architecture sets its own names)
     mixer_prefix: str = "mixer."
     feed_forward_prefix: str = "feed_forward."
@@ -147,7 +148,8 @@ class DecoderModel(Part):
             ff = make_part("feed_forward", layer.feed_forward.kind, prefix=layer.prefix + layer.feed_forward_prefix, **layer.feed_forward.kwargs())
             norm1 = make_part("norm", layer.mixer_norm.kind, prefix=layer.prefix + layer.mixer_norm_prefix, **layer.mixer_norm.kwargs())
             norm2 = make_part("norm", layer.ff_norm.kind, prefix=layer.prefix + layer.ff_norm_prefix, **layer.ff_norm.kwargs())
-            self.blocks.append(make_part("arrangement", layer.arrangement, prefix=layer.prefix, mixer=mixer, feed_forward=ff, mixer_norm=norm1, ff_norm=norm2))
+            self.blocks.append(make_part("arrangement", layer.arrangement, prefix=layer.prefix, mixer=mixer, feed_forward=ff, mixer_norm=norm1, ff_norm=norm2,
+                                         **dict(layer.arrangement_args)))
         self.final_norm = make_part("norm", spec.final_norm.kind, prefix=spec.final_norm_prefix, **spec.final_norm.kwargs())
         head = spec.head or PartSpec.of("linear")
         self.head = make_part("head", head.kind, name=spec.head_name, vocab_size=spec.vocab_size, hidden_size=spec.hidden_size,

@@ -12,7 +12,7 @@ from typing import Dict, Optional
 
 import torch
 
-from .base import DeferredNorm, Norm, Param, register_part, single
+from .base import DeferredNorm, Norm, Param, ResidualCopy, register_part, single
 
 
 class RMSNorm(Norm):
@@ -38,9 +38,14 @@ class RMSNorm(Norm):
             if delta.norm is not self or rows is not None:
                 raise ValueError("a DeferredNorm can only go to the norm it was made for, on all rows")
             return delta
+        if isinstance(delta, ResidualCopy):
+            delta = None  # (the block before has added everything itself)
         if rows is None:
             return ctx.ops.add_rmsnorm(residual, delta, self.weight, self.eps, ctx.dtype)
         return ctx.ops.add_rmsnorm_rows(residual, delta, rows, self.weight, self.eps, ctx.dtype)
+
+    def add_normed(self, residual, delta, mult, ctx):
+        return ctx.ops.norm_add(residual, delta, self.weight, self.eps, float(mult), ctx.dtype)
 
 
 register_part("norm", "rmsnorm", RMSNorm)

@@ -80,10 +80,33 @@ class RotaryEncoding(PositionEncoding):
         return self.cos, self.sin
 
 
+class SinusoidalEncoding(PositionEncoding):
+    """An absolute encoding added to the embeddings: entry ``2i`` of position ``p`` is ``sin(p * base^(-2i/width))`` and
+    entry ``2i + 1`` the cosine of the same angle.  Nothing is stored per position: the kernel takes the frequencies
+    (float64, built on the host) and works the angle out for each of the step's tokens, so there is no limit on
+    positions and no table of ``max_position x width``."""
+
+    def __init__(self, width: int, base: float = 10000.0) -> None:
+        super().__init__("")
+        if width < 1 or not base > 0:
+            raise ValueError("width and base must be positive")
+        self.width = int(width)
+        self.base = float(base)
+        self.frequencies: Optional[torch.Tensor] = None
+
+    def finalize(self, device, dtype) -> None:
+        pairs = (self.width + 1) // 2
+        self.frequencies = torch.tensor([self.base ** (-2.0 * i / self.width) for i in range(pairs)], dtype=torch.float64).to(device)
+
+    def on_embeddings(self, hidden: torch.Tensor, ctx) -> torch.Tensor:
+        return ctx.ops.add_sinusoid(hidden, ctx.positions, self.frequencies)
+
+
 class NoPositionEncoding(PositionEncoding):
     def __init__(self) -> None:
         super().__init__("")
 
 
 register_part("position", "rotary", RotaryEncoding)
+register_part("position", "sinusoidal", SinusoidalEncoding)
 register_part("position", "none", NoPositionEncoding)

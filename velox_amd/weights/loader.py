@@ -119,7 +119,7 @@ def named_tensors(model):
         row = 0
         for name, shape in zip(names, param.source_shapes):
             n = shape[0] if len(shape) > 0 else 1
-            piece = held[row:row + n].reshape(shape)
+            piece = held.reshape(shape) if held.dim() == 0 else held[row:row + n].reshape(shape)
             row += n
             if name not in seen and param.alias_of is None:
                 seen.add(name)
@@ -202,6 +202,9 @@ def bind(model, source, run_dtype: torch.dtype, device, ignore_unexpected: bool 
         target = torch.empty(param.shape, dtype=dtype, device=device)
         row = 0
         for piece in pieces:
+            if target.dim() == 0:  # (a single number, stored without a shape)
+                target.copy_(piece.to(dtype).reshape(()))
+                break
             n = piece.shape[0] if piece.dim() > 0 else 1
             target[row:row + n].copy_(piece.to(dtype))
             row += n
