@@ -31,6 +31,14 @@
 #endif
 
 constexpr int D = VELOX_HEAD_DIM;
+
+// Built with -DVELOX_ATTN_BIAS=1 the kernels add a bias by distance to the scaled scores: bias_table is float32
+// [heads, bias_len] and the key n positions behind the query reads column min(n, bias_len - 1) of the query head's row.
+// Without it the two arguments are ignored and the code is what it is without them.
+#ifndef VELOX_ATTN_BIAS
+#define VELOX_ATTN_BIAS 0
+#endif
+constexpr bool BIASED = VELOX_ATTN_BIAS != 0;
 static_assert(D % 16 == 0 && D >= 16 && D <= 256, "head size must be a multiple of 16 between 16 and 256");
 
 template <typename T> struct Frag;
@@ -144,7 +152,7 @@ __global__ void __launch_bounds__(64 * WAVES * KSPLIT) __attribute__((amdgpu_wav
     const T* __restrict__ qkv, int qkv_stride, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     const int* __restrict__ block_tables, int table_width, const int* __restrict__ cu_q, const int* __restrict__ kv_lens,
     T* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_lse,
-    int nh, int nkv, int page_shift, float scale, int window, int splits, int total_tokens) {
+    int nh, int nkv, int page_shift, float scale, int window, int splits, int total_tokens, const float* __restrict__ bias_table, int bias_len) {
   typedef Block<T> B;
   typedef typename B::Operand Operand;
   constexpr int KB = B::KB;
@@ -271,6 +279,7 @@ __global__ void __launch_bounds__(64 * WAVES * KSPLIT) __attribute__((amdgpu_wav
     for (int c = 0; c < NC; ++c) acc_o[ct][c] = float4_t{0.f, 0.f, 0.f, 0.f};
   }
   const float scale_eff = scale * Softmax<T>::SCALE;
+  const float scale_used = BIASED ? 1.f : scale_eff;  // (with a bias the scores are scaled where it is added)
 
   // ---- staging: global -> registers (issued a tile ahead) -> LDS; what does not change from tile to tile is computed once
   constexpr int VPR = D / VEC;              // vectors per key row of K
@@ -418,6 +427,31 @@ __global__ void __launch_bounds__(64 * WAVES * KSPLIT) __attribute__((amdgpu_wav
     }
     // ---- scale, mask (only where the tile crosses a row's limits), running maximum ----------
     const bool whole = n0 + BN <= kv_len && n0 + BN - 1 <= wave_first_pos && (window <= 0 || n0 > wave_last_pos - window);
+    if constexpr (BIASED) {
+      // the scores take their final form here (scaled, in the exponent's unit, bias added); a tile that lies wholly
+      // in the last column's reach gets one number per row
+#pragma unroll
+      for (int ct = 0; ct < CT; ++ct) {
+        const float* tab = bias_table + (size_t)head[ct] * bias_len;
+        const int d0 = pos[ct] - n0;  // distance of the tile's first key
+        if (d0 - (BN - 1) >= bias_len - 1) {
+          const float c = tab[bias_len - 1] * Softmax<T>::SCALE;
+#pragma unroll
+          for (int t = 0; t < NT; ++t)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) s[ct][t][j] = fmaf(s[ct][t][j], scale_eff, c);
+        } else {
+#pragma unroll
+          for (int t = 0; t < NT; ++t)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              int d = d0 - (16 * t + 4 * g + j);
+              d = d < 0 ? 0 : (d > bias_len - 1 ? bias_len - 1 : d);
+              s[ct][t][j] = fmaf(s[ct][t][j], scale_eff, tab[d] * Softmax<T>::SCALE);
+            }
+        }
+      }
+    }
     float alpha[CT];
     Operand pf[CT][NKB];
 #pragma unroll
@@ -442,7 +476,7 @@ __global__ void __launch_bounds__(64 * WAVES * KSPLIT) __attribute__((amdgpu_wav
       }
       mx = fmaxf(mx, __shfl_xor(mx, 16, VELOX_WAVE));
       mx = fmaxf(mx, __shfl_xor(mx, 32, VELOX_WAVE));
-      const float m_new = fmaxf(m_i[ct], mx * scale_eff);
+      const float m_new = fmaxf(m_i[ct], mx * scale_used);
       const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
       alpha[ct] = (m_i[ct] == -INFINITY) ? 0.f : Softmax<T>::exp_of(m_i[ct] - m_safe);
       float psum = 0.f;
@@ -455,7 +489,7 @@ __global__ void __launch_bounds__(64 * WAVES * KSPLIT) __attribute__((amdgpu_wav
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
             // a masked score is -inf and gives exp(-inf) = 0; m_safe is finite
-            const float p = Softmax<T>::exp_of(fmaf(s[ct][kb * TPB + u][j], scale_eff, -m_safe));
+            const float p = Softmax<T>::exp_of(fmaf(s[ct][kb * TPB + u][j], scale_used, -m_safe));
             psum += p;
             e[4 * u + j] = from_f32<T>(p);
           }
@@ -576,7 +610,7 @@ __global__ void __launch_bounds__(64 * WAVES * KSPLIT) __attribute__((amdgpu_wav
     const bf16_t* __restrict__ qkv, int qkv_stride, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int* __restrict__ block_tables, int table_width, const int* __restrict__ cu_q, const int* __restrict__ kv_lens,
     bf16_t* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_lse,
-    int nh, int nkv, int page_shift, float scale, int window, int splits, int total_tokens) {
+    int nh, int nkv, int page_shift, float scale, int window, int splits, int total_tokens, const float* __restrict__ bias_table, int bias_len) {
   typedef bf16_t T;
   typedef Block<T> B;
   typedef typename B::Operand Operand;
@@ -687,6 +721,7 @@ __global__ void __launch_bounds__(64 * WAVES * KSPLIT) __attribute__((amdgpu_wav
     for (int c = 0; c < NC; ++c) acc_o[ct][c] = float4_t{0.f, 0.f, 0.f, 0.f};
   }
   const float scale_eff = scale * Softmax<T>::SCALE;
+  const float scale_used = BIASED ? 1.f : scale_eff;  // (with a bias the scores are scaled where it is added)
 
   // ---- what each lane asks for: load instruction q = wave + WAVES * m of a tile fills bytes [1024 q, 1024 q + 1024) of
   // the K part (or the V^T part) of a buffer; lane l's 16 bytes are piece s = 64 q + l of the tile
@@ -827,6 +862,29 @@ __global__ void __launch_bounds__(64 * WAVES * KSPLIT) __attribute__((amdgpu_wav
     }
     // ---- scale, mask (only where the tile crosses a row's limits), running maximum ----------
     const bool whole = n0 + BN <= kv_len && n0 + BN - 1 <= wave_first_pos && (window <= 0 || n0 > wave_last_pos - window);
+    if constexpr (BIASED) {
+#pragma unroll
+      for (int ct = 0; ct < CT; ++ct) {
+        const float* tab = bias_table + (size_t)head[ct] * bias_len;
+        const int d0 = pos[ct] - n0;  // distance of the tile's first key
+        if (d0 - (BN - 1) >= bias_len - 1) {
+          const float c = tab[bias_len - 1] * Softmax<T>::SCALE;
+#pragma unroll
+          for (int t = 0; t < NT; ++t)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) s[ct][t][j] = fmaf(s[ct][t][j], scale_eff, c);
+        } else {
+#pragma unroll
+          for (int t = 0; t < NT; ++t)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              int d = d0 - (32 * (t >> 1) + 8 * g + 4 * (t & 1) + j);
+              d = d < 0 ? 0 : (d > bias_len - 1 ? bias_len - 1 : d);
+              s[ct][t][j] = fmaf(s[ct][t][j], scale_eff, tab[d] * Softmax<T>::SCALE);
+            }
+        }
+      }
+    }
     float alpha[CT];
     Operand pf[CT][NKB];
 #pragma unroll
@@ -856,7 +914,7 @@ __global__ void __launch_bounds__(64 * WAVES * KSPLIT) __attribute__((amdgpu_wav
       // exponent (powers of two): probabilities then stay below 2^REFERENCE_SLACK, far inside the range of both number
       // formats, and after a row's first tile the rescaling is the exception.
       constexpr float REFERENCE_SLACK = 8.f;
-      const float top = mx * scale_eff;
+      const float top = mx * scale_used;
       const bool stays = top - m_i[ct] <= REFERENCE_SLACK;  // (false while the row has seen no key: -inf)
       const float m_new = stays ? m_i[ct] : top;
       const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
@@ -870,7 +928,7 @@ __global__ void __launch_bounds__(64 * WAVES * KSPLIT) __attribute__((amdgpu_wav
         for (int u = 0; u < 2; ++u)
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
-            const float p = Softmax<T>::exp_of(fmaf(s[ct][kb * 2 + u][j], scale_eff, -m_safe));
+            const float p = Softmax<T>::exp_of(fmaf(s[ct][kb * 2 + u][j], scale_used, -m_safe));
             psum += p;
             e[4 * u + j] = from_f32<T>(p);
           }
@@ -1010,7 +1068,7 @@ __global__ void __launch_bounds__(64 * WAVES) decode_attention_kernel(
     const T* __restrict__ qkv, int qkv_stride, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     const int* __restrict__ block_tables, int table_width, const int* __restrict__ kv_lens,
     T* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_lse,
-    int nh, int nkv, int page_shift, float scale, int window, int splits, int total_tokens) {
+    int nh, int nkv, int page_shift, float scale, int window, int splits, int total_tokens, const float* __restrict__ bias_table, int bias_len) {
   constexpr int NC = D / 16;
   constexpr int NCW = (NC + WAVES - 1) / WAVES;
   typedef KeyOps<T, sizeof(T) == 2 && D % 32 == 0> KO;
@@ -1118,7 +1176,13 @@ __global__ void __launch_bounds__(64 * WAVES) decode_attention_kernel(
     for (int j = 0; j < 4; ++j) {
       const int n = n_begin + 16 * t + 4 * g + j;
       const bool keep = row_ok && n < kv_len && (window <= 0 || n > pos - window);
-      s[j] = keep ? s[j] * scale : -INFINITY;
+      if constexpr (BIASED) {
+        int d = pos - n;
+        d = d < 0 ? 0 : (d > bias_len - 1 ? bias_len - 1 : d);
+        s[j] = keep ? fmaf(s[j], scale, bias_table[(size_t)head * bias_len + d]) : -INFINITY;
+      } else {
+        s[j] = keep ? s[j] * scale : -INFINITY;
+      }
       mx = fmaxf(mx, s[j]);
     }
     mx = fmaxf(mx, __shfl_xor(mx, 16, VELOX_WAVE));
@@ -1265,7 +1329,7 @@ template <typename T>
 static int launch(const void* qkv, int qkv_stride, const void* k_cache, const void* v_cache, const int* block_tables, int table_width,
                   const int* cu_q, const int* kv_lens, void* out, float* part_o, float* part_lse, int num_seqs, int total_tokens,
                   int max_q_len, int max_kv_len, int nh, int nkv, int page_shift, float scale, int window, int splits, int first_token,
-                  hipStream_t stream) {
+                  const float* bias_table, int bias_len, hipStream_t stream) {
   constexpr int BN = tile_keys<T>();
   const int group = nh / nkv;
   // the streaming kernel keeps the page ids of a split's keys in LDS: they have to fit
@@ -1278,7 +1342,7 @@ static int launch(const void* qkv, int qkv_stride, const void* k_cache, const vo
     constexpr int DEPTH = sizeof(T) * D <= 256 ? 3 : 2;
     decode_attention_kernel<T, DEPTH, 4><<<dim3(splits, nkv, num_seqs), 256, 0, stream>>>(
         (const T*)qkv, qkv_stride, (const T*)k_cache, (const T*)v_cache, block_tables, table_width, kv_lens, (T*)out, part_o, part_lse,
-        nh, nkv, page_shift, scale, window, splits, total_tokens);
+        nh, nkv, page_shift, scale, window, splits, total_tokens, bias_table, bias_len);
     int status = (int)hipGetLastError();
     if (status != 0 || splits == 1) return status;
     merge_splits_kernel<T><<<dim3(total_tokens, nh), D < 64 ? 64 : D, 0, stream>>>(part_o, part_lse, (T*)out, nh, splits, total_tokens, 0);
@@ -1294,11 +1358,11 @@ static int launch(const void* qkv, int qkv_stride, const void* k_cache, const vo
       if (two_sets)
         direct_attention_kernel<2, 4, 2><<<grid, 512, 0, stream>>>(
             (const bf16_t*)qkv, qkv_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables, table_width, cu_q, kv_lens, (bf16_t*)out,
-            part_o, part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens);
+            part_o, part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens, bias_table, bias_len);
       else
         direct_attention_kernel<2, 4><<<grid, 256, 0, stream>>>(
             (const bf16_t*)qkv, qkv_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables, table_width, cu_q, kv_lens, (bf16_t*)out,
-            part_o, part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens);
+            part_o, part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens, bias_table, bias_len);
     }
     int status = (int)hipGetLastError();
     if (status != 0 || splits == 1) return status;
@@ -1356,29 +1420,29 @@ static int launch(const void* qkv, int qkv_stride, const void* k_cache, const vo
       if (rows >= 256 && workgroups * 4 >= 7LL * compute_units()) {
         paged_attention_kernel<T, BN, 2, 1, 4><<<grid, 256, 0, stream>>>(
             (const T*)qkv, qkv_stride, (const T*)k_cache, (const T*)v_cache, block_tables, table_width, cu_q, kv_lens, (T*)out, part_o,
-            part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens);
+            part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens, bias_table, bias_len);
       } else {
         paged_attention_kernel<T, BN, 1, 1, 8><<<grid, 512, 0, stream>>>(
             (const T*)qkv, qkv_stride, (const T*)k_cache, (const T*)v_cache, block_tables, table_width, cu_q, kv_lens, (T*)out, part_o,
-            part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens);
+            part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens, bias_table, bias_len);
       }
     } else {
       dim3 grid(num_seqs * splits, nkv, (rows + 255) / 256);
       paged_attention_kernel<T, BN, WIDE, 1, 8><<<grid, 512, 0, stream>>>(
           (const T*)qkv, qkv_stride, (const T*)k_cache, (const T*)v_cache, block_tables, table_width, cu_q, kv_lens, (T*)out, part_o,
-          part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens);
+          part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens, bias_table, bias_len);
     }
   } else if (WIDE == 2 && (long long)((rows + 63) / 64) * nkv * num_seqs * splits < 2 * compute_units() && max_kv_len >= 8 * BN) {
     // too few workgroups to fill the GPU and many keys each: two sets of waves share a workgroup's keys
     dim3 grid(num_seqs * splits, nkv, (rows + 63) / 64);
     paged_attention_kernel<T, BN, 1, WIDE><<<grid, 256 * WIDE, 0, stream>>>(
         (const T*)qkv, qkv_stride, (const T*)k_cache, (const T*)v_cache, block_tables, table_width, cu_q, kv_lens, (T*)out, part_o,
-        part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens);
+        part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens, bias_table, bias_len);
   } else {
     dim3 grid(num_seqs * splits, nkv, (rows + 63) / 64);
     paged_attention_kernel<T, BN, 1, 1><<<grid, 256, 0, stream>>>(
         (const T*)qkv, qkv_stride, (const T*)k_cache, (const T*)v_cache, block_tables, table_width, cu_q, kv_lens, (T*)out, part_o,
-        part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens);
+        part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens, bias_table, bias_len);
   }
   int status = (int)hipGetLastError();
   if (status != 0 || splits == 1) return status;
@@ -1388,6 +1452,7 @@ static int launch(const void* qkv, int qkv_stride, const void* k_cache, const vo
 }
 
 extern "C" int velox_attention_head_dim() { return D; }
+extern "C" int velox_attention_biased() { return BIASED ? 1 : 0; }
 
 // part_o: float32 [splits, total_tokens, nh, D]; part_lse: float32 [splits, total_tokens, nh]; both unused when splits == 1.
 // first_token: the sequences given (cu_q holds rows of qkv and out) cover rows [first_token, total_tokens); a launch for
@@ -1396,12 +1461,13 @@ extern "C" int velox_paged_attention(const void* qkv, int qkv_stride, const void
                                      const int* block_tables, int table_width, const int* cu_q, const int* kv_lens, void* out,
                                      float* part_o, float* part_lse, int num_seqs, int total_tokens, int max_q_len, int max_kv_len,
                                      int nh, int nkv, int page_shift, float scale, int window, int splits, int first_token, int dtype,
-                                     hipStream_t stream) {
+                                     const float* bias_table, int bias_len, hipStream_t stream) {
   if (num_seqs <= 0 || total_tokens <= 0) return 0;
+  if (BIASED ? (bias_table == nullptr || bias_len < 1) : bias_table != nullptr) return -1;  // (the build and the call must agree)
   if (nh % nkv != 0 || splits < 1 || page_shift < 0 || max_kv_len < 1 || first_token < 0 || first_token >= total_tokens) return -1;
   if (dtype == VELOX_BF16)
     return launch<bf16_t>(qkv, qkv_stride, k_cache, v_cache, block_tables, table_width, cu_q, kv_lens, out, part_o, part_lse, num_seqs,
-                          total_tokens, max_q_len, max_kv_len, nh, nkv, page_shift, scale, window, splits, first_token, stream);
+                          total_tokens, max_q_len, max_kv_len, nh, nkv, page_shift, scale, window, splits, first_token, bias_table, bias_len, stream);
   return launch<float>(qkv, qkv_stride, k_cache, v_cache, block_tables, table_width, cu_q, kv_lens, out, part_o, part_lse, num_seqs,
-                       total_tokens, max_q_len, max_kv_len, nh, nkv, page_shift, scale, window, splits, first_token, stream);
+                       total_tokens, max_q_len, max_kv_len, nh, nkv, page_shift, scale, window, splits, first_token, bias_table, bias_len, stream);
 }

@@ -93,4 +93,13 @@ __device__ __forceinline__ void load4(const T* __restrict__ base, size_t row_off
   }
 }
 
+// The middle of a gated unit: g sigmoid(alpha g) (u + shift) with g = min(gate, limit), u = clamp(up, -limit, limit);
+// (1, inf, 0) is silu(gate) * up.
+struct GluUnit { float alpha, limit, shift; };
+__device__ __forceinline__ float glu_middle(float gate, float up, const GluUnit& unit) {
+  const float g = fminf(gate, unit.limit);
+  const float u = fminf(fmaxf(up, -unit.limit), unit.limit);
+  return g / (1.f + expf(-unit.alpha * g)) * (u + unit.shift);
+}
+
 #define VELOX_RETURN_LAUNCH_STATUS() return (int)hipGetLastError()

@@ -41,6 +41,7 @@ struct GroupedArgs {
   const bf16_t* gate;  // GM_GATE: times sigmoid(gate[r * gate_ld + g * n + col])
   long long gate_ld;
   const float* row_scale;  // GM_ROW_SCALE: times row_scale[order[r]]
+  GluUnit unit = {1.f, INFINITY, 0.f};  // GM_GLU: the unit's middle (see glu_middle)
 };
 
 __device__ __forceinline__ gm_bf16x8_t gm_load(const bf16_t* p, bool ok) {
@@ -171,7 +172,7 @@ __global__ void __launch_bounds__(256) grouped_mfma_kernel(const GroupedArgs arg
         const int col = col0[t] + 4 * g4 + j;
         if (col >= n) continue;
         float v = acc[t][mt][j];
-        if (EPI == GM_GLU) v = v / (1.f + expf(-v)) * acc[t + GM_NT / 2][mt][j];
+        if (EPI == GM_GLU) v = glu_middle(v, acc[t + GM_NT / 2][mt][j], args.unit);
         if (EPI == GM_GATE) {
           const float z = to_f32(args.gate[(size_t)(row0 + r) * args.gate_ld + (size_t)group * n + col]);
           v *= 1.f / (1.f + expf(-z));
@@ -279,7 +280,7 @@ __global__ void __launch_bounds__(256) grouped_mfma_few_rows_kernel(const Groupe
         const int col = col0[t] + 4 * g4 + j;
         if (col >= n) continue;
         float v = acc[t][mt][j];
-        if (EPI == GM_GLU) v = v / (1.f + expf(-v)) * acc[1][mt][j];
+        if (EPI == GM_GLU) v = glu_middle(v, acc[1][mt][j], args.unit);
         if (EPI == GM_GATE) {
           const float z = to_f32(args.gate[(size_t)(row0 + r) * args.gate_ld + (size_t)group * n + col]);
           v *= 1.f / (1.f + expf(-z));

@@ -25,12 +25,13 @@
 // route_top: one wave per token, its lanes over the experts.  score = sigmoid(z) or softmax(z) over all experts; the `top`
 // largest scores, ties to the lower index; weights are the chosen scores, divided by their sum when `renormalize`.
 // Every round the wave takes the largest score that is not yet taken (value first, then the lower index), so the choices
-// come out in descending order of score.
+// come out in descending order of score.  With `correction` (float32 [experts]) the choice goes by score + correction and
+// the weights stay the scores themselves.
 // ---------------------------------------------------------------------------------------------
 #define ROUTE_PER_LANE 32  // experts per lane held in registers: up to 2,048 experts
 
 __global__ void __launch_bounds__(256) route_top_kernel(const float* __restrict__ logits, int* __restrict__ choice, float* __restrict__ weight, int tokens,
-                                                        int experts, int top, int softmax, int renormalize) {
+                                                        int experts, int top, int softmax, int renormalize, const float* __restrict__ correction) {
   const int lane = threadIdx.x & 63;
   const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (t >= tokens) return;  // (a whole wave; nothing below crosses waves)
@@ -48,12 +49,15 @@ __global__ void __launch_bounds__(256) route_top_kernel(const float* __restrict_
 #pragma unroll
   for (int u = 0; u < ROUTE_PER_LANE; ++u) {
     const int e = lane + 64 * u;
-    score[u] = -1.f;  // (scores are positive: -1 marks "no such expert" and "taken")
-    if (e < experts) score[u] = softmax ? expf(z[e] - shift) / denom : 1.f / (1.f + expf(-z[e]));
+    score[u] = -INFINITY;  // ("no such expert" and "taken")
+    if (e < experts) {
+      score[u] = softmax ? expf(z[e] - shift) / denom : 1.f / (1.f + expf(-z[e]));
+      if (correction) score[u] += correction[e];
+    }
   }
   float total = 0.f;
   for (int k = 0; k < top; ++k) {
-    float best = -1.f;
+    float best = -INFINITY;
     int best_e = 0x7fffffff;
 #pragma unroll
     for (int u = 0; u < ROUTE_PER_LANE; ++u)
@@ -66,7 +70,10 @@ __global__ void __launch_bounds__(256) route_top_kernel(const float* __restrict_
     }
 #pragma unroll
     for (int u = 0; u < ROUTE_PER_LANE; ++u)
-      if (lane + 64 * u == best_e) score[u] = -1.f;
+      if (lane + 64 * u == best_e) score[u] = -INFINITY;
+    // (the weight is the score without the correction: the same expression as above, so the same value)
+    if (best_e >= experts) best_e = 0;  // (only when every score left is a NaN: stay inside the row)
+    if (correction) best = softmax ? expf(z[best_e] - shift) / denom : 1.f / (1.f + expf(-z[best_e]));
     total += best;
     if (lane == 0) {
       choice[(size_t)t * top + k] = best_e;
@@ -78,10 +85,10 @@ __global__ void __launch_bounds__(256) route_top_kernel(const float* __restrict_
 }
 
 extern "C" int velox_route_top(const float* logits, int* choice, float* weight, int tokens, int experts, int top, int softmax, int renormalize,
-                               hipStream_t stream) {
+                               const float* correction, hipStream_t stream) {
   if (tokens <= 0) return 0;
   if (experts < 1 || experts > 64 * ROUTE_PER_LANE || top < 1 || top > experts) return -1;
-  route_top_kernel<<<(tokens + 3) / 4, 256, 0, stream>>>(logits, choice, weight, tokens, experts, top, softmax, renormalize);
+  route_top_kernel<<<(tokens + 3) / 4, 256, 0, stream>>>(logits, choice, weight, tokens, experts, top, softmax, renormalize, correction);
   VELOX_RETURN_LAUNCH_STATUS();
 }
 
@@ -186,7 +193,7 @@ extern "C" int velox_routed_plan(const int* choice, int pairs, int experts, int*
 template <typename T, typename TO, bool GLU>
 __global__ void __launch_bounds__(256) grouped_product_kernel(const T* __restrict__ a, const T* __restrict__ w, TO* __restrict__ out,
                                                               const int* __restrict__ plan, const float* __restrict__ pair_weight, int pairs, int experts,
-                                                              int max_tiles, int top, int n, int k, int scale_rows, int a_vec, int w_vec) {
+                                                              int max_tiles, int top, int n, int k, int scale_rows, int a_vec, int w_vec, GluUnit unit) {
   __shared__ float a_tile[RT_BK][RT_BM + RT_PAD];
   __shared__ float w_tile[GLU ? 2 : 1][RT_BK][RT_BN + RT_PAD];
   __shared__ int row_pair[RT_BM];
@@ -284,7 +291,7 @@ __global__ void __launch_bounds__(256) grouped_product_kernel(const T* __restric
       float v = total[0][i][j] + acc[0][i][j];
       if (GLU) {
         const float up = total[NW - 1][i][j] + acc[NW - 1][i][j];
-        v = v / (1.f + expf(-v)) * up;  // (float32 throughout, one rounding at the store)
+        v = glu_middle(v, up, unit);  // (float32 throughout, one rounding at the store)
       } else {
         v *= row_scale;
       }
@@ -294,8 +301,9 @@ __global__ void __launch_bounds__(256) grouped_product_kernel(const T* __restric
 }
 
 extern "C" int velox_grouped_glu(const void* x, const void* gate_up, void* act, const int* plan, const float* pair_weight, int pairs, int experts, int top,
-                                 int inter, int hidden, int scale_input, int dtype, hipStream_t stream) {
+                                 int inter, int hidden, int scale_input, int dtype, float alpha, float limit, float shift, hipStream_t stream) {
   if (pairs <= 0) return 0;
+  const GluUnit unit = {alpha, limit, shift};
   const int max_tiles = velox_routed_max_tiles(pairs, experts);
   dim3 grid((inter + RT_BN - 1) / RT_BN, max_tiles);
   if (grid.y > 65535) return -1;
@@ -304,10 +312,10 @@ extern "C" int velox_grouped_glu(const void* x, const void* gate_up, void* act, 
   const int w_vec = hidden % 4 == 0 && ((uintptr_t)gate_up) % (4 * size) == 0;
   if (dtype == VELOX_BF16)
     grouped_product_kernel<bf16_t, bf16_t, true><<<grid, 256, 0, stream>>>((const bf16_t*)x, (const bf16_t*)gate_up, (bf16_t*)act, plan, pair_weight, pairs, experts,
-                                                                           max_tiles, top, inter, hidden, scale_input, a_vec, w_vec);
+                                                                           max_tiles, top, inter, hidden, scale_input, a_vec, w_vec, unit);
   else
     grouped_product_kernel<float, float, true><<<grid, 256, 0, stream>>>((const float*)x, (const float*)gate_up, (float*)act, plan, pair_weight, pairs, experts,
-                                                                         max_tiles, top, inter, hidden, scale_input, a_vec, w_vec);
+                                                                         max_tiles, top, inter, hidden, scale_input, a_vec, w_vec, unit);
   VELOX_RETURN_LAUNCH_STATUS();
 }
 
@@ -322,10 +330,10 @@ extern "C" int velox_grouped_down(const void* act, const void* down, float* y, c
   const int w_vec = inter % 4 == 0 && ((uintptr_t)down) % (4 * size) == 0;
   if (dtype == VELOX_BF16)
     grouped_product_kernel<bf16_t, float, false><<<grid, 256, 0, stream>>>((const bf16_t*)act, (const bf16_t*)down, y, plan, pair_weight, pairs, experts, max_tiles,
-                                                                           top, hidden, inter, scale_output, a_vec, w_vec);
+                                                                           top, hidden, inter, scale_output, a_vec, w_vec, GluUnit{1.f, INFINITY, 0.f});
   else
     grouped_product_kernel<float, float, false><<<grid, 256, 0, stream>>>((const float*)act, (const float*)down, y, plan, pair_weight, pairs, experts, max_tiles,
-                                                                          top, hidden, inter, scale_output, a_vec, w_vec);
+                                                                          top, hidden, inter, scale_output, a_vec, w_vec, GluUnit{1.f, INFINITY, 0.f});
   VELOX_RETURN_LAUNCH_STATUS();
 }
 
@@ -334,8 +342,9 @@ extern "C" int velox_grouped_down(const void* act, const void* down, float* y, c
 // weight scales the expert's input: float32 product, one rounding), then both grouped products read sorted rows.
 // ---------------------------------------------------------------------------------------------
 __global__ void __launch_bounds__(256) routed_gather_kernel(const bf16_t* __restrict__ x, const int* __restrict__ order, const float* __restrict__ pair_weight,
-                                                            bf16_t* __restrict__ sorted, int top, int hidden, int scale) {
+                                                            bf16_t* __restrict__ sorted, int top, int hidden, int scale, const int* __restrict__ placed) {
   const int row = blockIdx.x;
+  if (row >= *placed) return;  // (pairs whose expert the plan leaves out have no row: `order` ends at the placed ones)
   const int pair = order[row];
   const bf16_t* src = x + (size_t)(pair / top) * hidden;
   bf16_t* dst = sorted + (size_t)row * hidden;
@@ -364,15 +373,16 @@ static GroupedArgs routed_args(const void* a, const void* w, void* out, const in
 // inter % 8 == 0 (the caller checks).
 extern "C" int velox_routed_products_bf16(const void* x, const void* gate_up, const void* down, void* sorted, void* act, float* y, const int* plan,
                                           const float* pair_weight, int pairs, int experts, int top, int inter, int hidden, int scale_input,
-                                          int tile_rows, hipStream_t stream) {
+                                          int tile_rows, float alpha, float limit, float shift, hipStream_t stream) {
   if (pairs <= 0) return 0;
   if (hidden % 8 != 0 || inter % 8 != 0) return -1;
   const int max_tiles = velox_routed_max_tiles(pairs, experts);
   if (max_tiles > 65535) return -1;
   const int* order = plan + 1 + (experts + 1);
   if (x != nullptr)  // (nullptr: the plan kernel has copied the rows already)
-    routed_gather_kernel<<<pairs, 256, 0, stream>>>((const bf16_t*)x, order, pair_weight, (bf16_t*)sorted, top, hidden, scale_input);
+    routed_gather_kernel<<<pairs, 256, 0, stream>>>((const bf16_t*)x, order, pair_weight, (bf16_t*)sorted, top, hidden, scale_input, plan + 1 + experts);
   GroupedArgs glu = routed_args(sorted, gate_up, act, plan, pairs, experts, inter, hidden, 2 * inter);
+  glu.unit = GluUnit{alpha, limit, shift};
   grouped_mfma_launch<GM_GLU, bf16_t>(glu, pairs, tile_rows, max_tiles, 1, stream);
   GroupedArgs last = routed_args(act, down, y, plan, pairs, experts, hidden, inter, hidden);
   last.row_scale = pair_weight;
@@ -383,10 +393,13 @@ extern "C" int velox_routed_products_bf16(const void* x, const void* gate_up, co
 
 // ---------------------------------------------------------------------------------------------
 // out[t, :] = (sum_k y[place[t * top + k], :]) + shared[t, :], the choices added in order, one rounding at the store.
+// With `x`: a choice that the plan has not placed (an identity expert, whose index lies behind the real ones) adds
+// pair_weight[t * top + k] * x[t, :] in its turn.
 // ---------------------------------------------------------------------------------------------
 template <typename T>
 __global__ void __launch_bounds__(256) routed_combine_kernel(const float* __restrict__ y, const int* __restrict__ place, const T* __restrict__ shared,
-                                                             T* __restrict__ out, int top, int hidden) {
+                                                             T* __restrict__ out, int top, int hidden, const T* __restrict__ x,
+                                                             const float* __restrict__ pair_weight) {
   __shared__ int rows[64];  // the token's rows of y, looked up once (up to 64 choices; more are looked up as they are added)
   const int t = blockIdx.x;
   const int* mine = place + (size_t)t * top;
@@ -400,6 +413,7 @@ __global__ void __launch_bounds__(256) routed_combine_kernel(const float* __rest
     for (int k = 0; k < top; ++k) {
       const int row = mine[k];
       if (row >= 0) v += y[(size_t)row * hidden + i];
+      else if (x) v += pair_weight[(size_t)t * top + k] * to_f32(x[(size_t)t * hidden + i]);
     }
     if (shared) v += to_f32(shared[(size_t)t * hidden + i]);
     out[(size_t)t * hidden + i] = from_f32<T>(v);
@@ -407,12 +421,12 @@ __global__ void __launch_bounds__(256) routed_combine_kernel(const float* __rest
 }
 
 extern "C" int velox_routed_combine(const float* y, const int* plan, const void* shared, void* out, int tokens, int top, int experts, int hidden, int dtype,
-                                    hipStream_t stream) {
+                                    const void* x, const float* pair_weight, hipStream_t stream) {
   if (tokens <= 0) return 0;
   const int* place = plan + 1 + (experts + 1) + (size_t)tokens * top;
   if (dtype == VELOX_BF16)
-    routed_combine_kernel<bf16_t><<<tokens, 256, 0, stream>>>(y, place, (const bf16_t*)shared, (bf16_t*)out, top, hidden);
+    routed_combine_kernel<bf16_t><<<tokens, 256, 0, stream>>>(y, place, (const bf16_t*)shared, (bf16_t*)out, top, hidden, (const bf16_t*)x, pair_weight);
   else
-    routed_combine_kernel<float><<<tokens, 256, 0, stream>>>(y, place, (const float*)shared, (float*)out, top, hidden);
+    routed_combine_kernel<float><<<tokens, 256, 0, stream>>>(y, place, (const float*)shared, (float*)out, top, hidden, (const float*)x, pair_weight);
   VELOX_RETURN_LAUNCH_STATUS();
 }

@@ -53,7 +53,7 @@ class Replayer:
         capacity = pages * block_size
         self.max_model_len = min(capacity, model_position_limit(self.config))
         self.model = build_model(self.config, self.dtype, self.device, max_position=self.max_model_len)
-        bind_from_checkpoint(self.model, model_dir, self.dtype, self.device)
+        bind_from_checkpoint(self.model, model_dir, self.dtype, self.device, ignore_unexpected=True)  # (tensors the model has no place for are counted and left)
         ops.prepare(self.model, self.dtype)
         self.cache = CacheManager(self.model.cache_needs(), block_size, pages + 1, max_live, self.dtype, self.device, max_model_len=self.max_model_len)
         self.runner = ModelRunner(self.model, self.cache, ops, self.dtype, self.device, max_num_tokens=max(capacity, 64), max_num_seqs=max_live, enable_graphs=enable_graphs)

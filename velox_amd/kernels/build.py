@@ -23,11 +23,13 @@ SOURCE_DIR = os.path.join(PACKAGE_DIR, "csrc")
 ARCH = "gfx950"
 # hipcc -O3 must not form packed float32 operations from scalar code on this target
 FLAGS = ["-O3", f"--offload-arch={ARCH}", "-shared", "-fPIC", "-std=c++17", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
-CORE_SOURCES = ["elementwise.hip", "gemm.hip", "skinny_gemm.hip", "latent.hip", "routed.hip", "sampling.hip", "probe.hip"]
+CORE_SOURCES = ["elementwise.hip", "gemm.hip", "skinny_gemm.hip", "latent.hip", "routed.hip", "normed.hip", "sampling.hip", "probe.hip"]
 ATTENTION_SOURCES = ["attention.hip"]
 HEADERS = ["common.h", "no_alloc.h", "grouped_mfma.h"]
 # head sizes built ahead of time by build_all(); any other multiple of 16 up to 256 is built at first use
 DEFAULT_HEAD_DIMS = (16, 32, 48, 64, 80, 96, 128, 192, 256)
+# the same kernels with a bias by distance on the scores (``attnbias_d<N>``), built ahead of time for these head sizes
+DEFAULT_BIASED_HEAD_DIMS = (16, 32, 48, 64, 128)
 
 
 class BuildError(RuntimeError):
@@ -159,16 +161,25 @@ def ensure_core(force: bool = False) -> str:
     return ensure_library("core", CORE_SOURCES, {}, force)
 
 
-def ensure_attention(head_dim: int, force: bool = False) -> str:
+def _attention_job(head_dim: int, biased: bool):
+    # (the two stems share no prefix: a new build of one removes the stale files of its own stem only)
+    if biased:
+        return f"attnbias_d{head_dim}", ATTENTION_SOURCES, {"VELOX_HEAD_DIM": head_dim, "VELOX_ATTN_BIAS": 1}
+    return f"attn_d{head_dim}", ATTENTION_SOURCES, {"VELOX_HEAD_DIM": head_dim}
+
+
+def ensure_attention(head_dim: int, force: bool = False, biased: bool = False) -> str:
+    """``biased``: the build whose scores take a bias by distance."""
     if head_dim % 16 != 0 or not 16 <= head_dim <= 256:
         raise BuildError(f"head_dim={head_dim}: the attention kernels take multiples of 16 from 16 to 256")
-    return ensure_library(f"attn_d{head_dim}", ATTENTION_SOURCES, {"VELOX_HEAD_DIM": head_dim}, force)
+    stem, sources, defines = _attention_job(head_dim, biased)
+    return ensure_library(stem, sources, defines, force)
 
 
-def build_all(head_dims: Sequence[int] = DEFAULT_HEAD_DIMS, force: bool = True) -> List[str]:
+def build_all(head_dims: Sequence[int] = DEFAULT_HEAD_DIMS, force: bool = True, biased_head_dims: Sequence[int] = DEFAULT_BIASED_HEAD_DIMS) -> List[str]:
     """Compiles every library (in parallel, one hipcc per library)."""
     from concurrent.futures import ThreadPoolExecutor
 
-    jobs = [("core", CORE_SOURCES, {})] + [(f"attn_d{d}", ATTENTION_SOURCES, {"VELOX_HEAD_DIM": d}) for d in head_dims]
+    jobs = [("core", CORE_SOURCES, {})] + [_attention_job(d, False) for d in head_dims] + [_attention_job(d, True) for d in biased_head_dims]
     with ThreadPoolExecutor(max_workers=min(8, len(jobs))) as pool:
         return list(pool.map(lambda job: ensure_library(job[0], job[1], job[2], force), jobs))

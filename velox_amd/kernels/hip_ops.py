@@ -91,7 +91,7 @@ class HipOps:
         if arch != build.ARCH:
             raise KernelError(f"the kernels are built for {build.ARCH}; this GPU is {arch}")
         self._core = ctypes.CDLL(build.ensure_core())
-        self._attention: Dict[int, ctypes.CDLL] = {}
+        self._attention: Dict[Tuple[int, bool], ctypes.CDLL] = {}
         self._declare_core()
         self.num_cus = torch.cuda.get_device_properties(self.device).multi_processor_count
         self.use_library_gemm = True
@@ -144,35 +144,44 @@ class HipOps:
         c.velox_head_linear.argtypes = [_P, _I, _I, _I, _P, _P, _I, _I, _I, _P, _I, _I, _I, _I, _I, _I, _I, _P]
         c.velox_plain_attention.argtypes = [_P, _I, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _P]
         c.velox_plain_attention.restype = _I
-        c.velox_route_top.argtypes = [_P, _P, _P, _I, _I, _I, _I, _I, _P]
+        c.velox_route_top.argtypes = [_P, _P, _P, _I, _I, _I, _I, _I, _P, _P]
         c.velox_routed_plan_elems.argtypes = [_I, _I]
         c.velox_routed_plan_elems.restype = ctypes.c_longlong
         c.velox_routed_plan.argtypes = [_P, _I, _I, _P, _I, _P, _P, _P, _I, _I, _I, _P]
-        c.velox_grouped_glu.argtypes = [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P]
+        c.velox_grouped_glu.argtypes = [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _F, _F, _P]
         c.velox_grouped_down.argtypes = [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P]
-        c.velox_routed_combine.argtypes = [_P, _P, _P, _P, _I, _I, _I, _I, _I, _P]
-        c.velox_routed_products_bf16.argtypes = [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P]
+        c.velox_routed_combine.argtypes = [_P, _P, _P, _P, _I, _I, _I, _I, _I, _P, _P, _P]
+        c.velox_routed_products_bf16.argtypes = [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _F, _F, _P]
+        c.velox_add_sinusoid.argtypes = [_P, _P, _P, _I, _I, _P]
+        c.velox_add_cast.argtypes = [_P, _P, _I, _P, ctypes.c_longlong, _P]
+        c.velox_norm_add.argtypes = [_P, _P, _I, _P, _P, _I, _I, _F, _F, _I, ctypes.c_longlong, _P]
+        c.velox_qk_norm_write.argtypes = [_P, _I, _P, _P, _P, _P, _P, _I, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _F, _F, _I, _I, _P]
         c.velox_routed_products_bf16.restype = _I
         for fn in (c.velox_latent_rotate_write, c.velox_head_linear, c.velox_route_top, c.velox_routed_plan, c.velox_grouped_glu, c.velox_grouped_down,
-                   c.velox_routed_combine):
+                   c.velox_routed_combine, c.velox_add_sinusoid, c.velox_add_cast, c.velox_norm_add, c.velox_qk_norm_write):
             fn.restype = _I
         for fn in (c.velox_embed, c.velox_place_tokens, c.velox_add_rmsnorm, c.velox_silu_mul, c.velox_rope_kv_write, c.velox_gemm_fma,
                    c.velox_argmax, c.velox_sample, c.velox_sample_chunked, c.velox_apply_penalties, c.velox_count_tokens, c.velox_count_sampled,
                    c.velox_penalties_from_counts):
             fn.restype = _I
 
-    def attention_library(self, head_dim: int) -> ctypes.CDLL:
-        lib = self._attention.get(head_dim)
+    def attention_library(self, head_dim: int, biased: bool = False) -> ctypes.CDLL:
+        """The attention kernels for one head size; ``biased``: the build whose scores take a bias by distance."""
+        key = (head_dim, bool(biased))
+        lib = self._attention.get(key)
         if lib is None:
-            lib = ctypes.CDLL(build.ensure_attention(head_dim))
-            lib.velox_paged_attention.argtypes = [_P, _I, _P, _P, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I, _I, _P]
+            lib = ctypes.CDLL(build.ensure_attention(head_dim, biased=bool(biased)))
+            lib.velox_paged_attention.argtypes = [_P, _I, _P, _P, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I, _I, _P, _I, _P]
+            lib.velox_attention_biased.restype = _I
             lib.velox_paged_attention.restype = _I
             lib.velox_attention_head_dim.restype = _I
             lib.velox_attention_portion_kernel.argtypes = [_I]
             lib.velox_attention_portion_kernel.restype = None
             if lib.velox_attention_head_dim() != head_dim:
                 raise KernelError(f"attention library for head_dim={head_dim} reports {lib.velox_attention_head_dim()}")
-            self._attention[head_dim] = lib
+            if bool(lib.velox_attention_biased()) != bool(biased):
+                raise KernelError(f"attention library for head_dim={head_dim}: built {'with' if lib.velox_attention_biased() else 'without'} the bias by distance")
+            self._attention[key] = lib
         return lib
 
     def prepare(self, model, dtype) -> None:
@@ -362,6 +371,91 @@ class HipOps:
 
     def add_rmsnorm_rows(self, residual, delta, rows, weight, eps, out_dtype):
         return self._norm(residual, delta, rows, weight, eps, out_dtype)
+
+    def add_sinusoid(self, hidden: torch.Tensor, positions: torch.Tensor, frequencies: torch.Tensor) -> torch.Tensor:
+        """``hidden[t, 2i] += sin(p_t f_i)``, ``hidden[t, 2i + 1] += cos(p_t f_i)`` in place; ``frequencies`` float64 [ceil(H / 2)]."""
+        self._check("hidden", hidden, torch.float32)
+        if hidden.dim() != 2:
+            raise KernelError("add_sinusoid: hidden must be [T, H]")
+        tokens, width = hidden.shape
+        self._check("positions", positions, torch.int32, (tokens,))
+        self._check("frequencies", frequencies, torch.float64, ((width + 1) // 2,), align=8)
+        self._launched(self._core.velox_add_sinusoid(_ptr(hidden), _ptr(positions), _ptr(frequencies), tokens, width, self._stream()), "add_sinusoid")
+        return hidden
+
+    def add_cast(self, residual: torch.Tensor, delta: Optional[torch.Tensor], out_dtype: torch.dtype) -> torch.Tensor:
+        """``residual += delta`` in place (``delta`` may be None) and the residual in ``out_dtype`` (itself when that is float32)."""
+        self._check("residual", residual, torch.float32)
+        if delta is not None:
+            self._check("delta", delta, None, tuple(residual.shape))
+        if delta is None and out_dtype == torch.float32:
+            return residual
+        out = torch.empty_like(residual, dtype=out_dtype) if out_dtype != torch.float32 else None
+        self._launched(self._core.velox_add_cast(_ptr(residual), _ptr(delta), _code(delta.dtype) if delta is not None else 0, _ptr(out), residual.numel(),
+                                                 self._stream()), "add_cast")
+        return residual if out is None else out
+
+    def norm_add(self, residual: torch.Tensor, delta: torch.Tensor, weight: torch.Tensor, eps: float, mult: float, out_dtype: torch.dtype) -> torch.Tensor:
+        """``residual += mult * delta * rsqrt(mean(delta^2) + eps) * weight`` in place, float32 throughout; ``delta`` is [T, H]
+        or float32 partial sums [S, T, H], added first to last.  Returns the residual in ``out_dtype`` (itself when float32)."""
+        self._check("residual", residual, torch.float32)
+        if residual.dim() != 2:
+            raise KernelError("norm_add: residual must be [T, H]")
+        tokens, hidden = residual.shape
+        self._check("weight", weight, torch.float32, (hidden,))
+        partials, partial_stride = 1, 0
+        if delta.dim() == 3:
+            partials, partial_stride = delta.shape[0], tokens * hidden
+            self._check("delta", delta, torch.float32, (partials, tokens, hidden))
+        else:
+            self._check("delta", delta, None, (tokens, hidden))
+        out = torch.empty((tokens, hidden), dtype=out_dtype, device=self.device) if out_dtype != torch.float32 else None
+        self._launched(self._core.velox_norm_add(_ptr(residual), _ptr(delta), _code(delta.dtype), _ptr(weight), _ptr(out), tokens, hidden, float(eps), float(mult),
+                                                 partials, partial_stride, self._stream()), "norm_add")
+        return residual if out is None else out
+
+    def qk_norm_write(self, qkv, num_heads, num_kv_heads, dim, vdim, cached_dim, q_norm, k_norm, whole, eps, q_temp, positions, first_values, mix_weight,
+                      slot_mapping, k_cache, v_cache, block_size, write_kv=True) -> torch.Tensor:
+        """Rows of ``qkv`` hold ``num_heads`` queries and ``num_kv_heads`` keys of ``dim`` channels and ``num_kv_heads`` values
+        of ``vdim``.  Queries and keys pass an RMS norm (``whole``: over all heads at once, weights of that size; else per head
+        with one weight of ``dim``), the queries the temperature ``q_temp = (coef, every)``; values are blended with
+        ``first_values = (tensor, first column)`` by ``mix_weight`` (one float32 on the device).  Returns the queries as the
+        attention kernels read them, ``[T, num_heads * cached_dim]``; keys and values go into the cache at that head size,
+        padding channels as zeros."""
+        if qkv.dim() != 2:
+            raise KernelError("qk_norm_write: rows are [T, width]")
+        tokens, width = qkv.shape
+        q_size, k_size, v_size = num_heads * dim, num_kv_heads * dim, num_kv_heads * vdim
+        self._check("qkv", qkv, None, (tokens, q_size + k_size + v_size))
+        self._check("positions", positions, torch.int32, (tokens,))
+        self._check("q_norm", q_norm, torch.float32, (q_size if whole else dim,))
+        self._check("k_norm", k_norm, torch.float32, (k_size if whole else dim,))
+        if cached_dim < max(dim, vdim) or block_size <= 0 or block_size & (block_size - 1):
+            raise KernelError(f"qk_norm_write: cached_dim={cached_dim} below dim={dim} or vdim={vdim}, or block_size={block_size} no power of two")
+        first = first_offset = first_stride = None
+        if first_values is not None:
+            first, first_offset = first_values
+            self._check("first_values", first, qkv.dtype)
+            if first.dim() != 2 or first.shape[0] != tokens or first_offset < 0 or first_offset + v_size > first.shape[1]:
+                raise KernelError("qk_norm_write: the earlier layer's values do not lie inside the rows given")
+            first_stride = first.shape[1]
+            self._check("mix_weight", mix_weight, torch.float32, ())
+        if write_kv:
+            self._check("slot_mapping", slot_mapping, torch.int32, (tokens,))
+            pages = k_cache.shape[0]
+            self._check("k_cache", k_cache, qkv.dtype, (pages, num_kv_heads, block_size, cached_dim))
+            self._check("v_cache", v_cache, qkv.dtype, (pages, num_kv_heads, cached_dim, block_size))
+        coef, every = (float(q_temp[0]), int(q_temp[1])) if q_temp is not None else (0.0, 0)
+        if q_temp is not None and every < 1:
+            raise KernelError("qk_norm_write: q_temp's 'every' must be at least 1")
+        queries = torch.empty((tokens, num_heads * cached_dim), dtype=qkv.dtype, device=self.device)
+        status = self._core.velox_qk_norm_write(
+            _ptr(qkv), width, _ptr(queries), _ptr(q_norm), _ptr(k_norm), _ptr(positions), _ptr(first), int(first_stride or 0), int(first_offset or 0),
+            _ptr(mix_weight) if first is not None else _P(0), _ptr(slot_mapping) if write_kv else _P(0), _ptr(k_cache) if write_kv else _P(0),
+            _ptr(v_cache) if write_kv else _P(0), tokens, num_heads, num_kv_heads, dim, vdim, cached_dim, block_size.bit_length() - 1, int(bool(whole)),
+            int(bool(write_kv)), float(eps), coef, every, _code(qkv.dtype), self._stream())
+        self._launched(status, "qk_norm_write")
+        return queries
 
     # -- matrix products --------------------------------------------------------------------------
     @staticmethod
@@ -811,28 +905,38 @@ class HipOps:
         return out
 
     # -- routed experts ---------------------------------------------------------------------------
-    def route_top(self, logits: torch.Tensor, top: int, score: str = "sigmoid", renormalize: bool = False):
+    def route_top(self, logits: torch.Tensor, top: int, score: str = "sigmoid", renormalize: bool = False, correction: Optional[torch.Tensor] = None):
         """float32 ``logits`` [T, E] -> (int32 choices [T, top], float32 weights [T, top]): the ``top`` largest scores
-        (``sigmoid`` or ``softmax`` over all experts), ties to the lower index, divided by their sum when ``renormalize``."""
+        (``sigmoid`` or ``softmax`` over all experts), ties to the lower index, divided by their sum when ``renormalize``.
+        ``correction`` (float32 [E]) is added to the scores for the choice only: the weights are the scores without it."""
         self._check("logits", logits, torch.float32)
+        if correction is not None:
+            self._check("correction", correction, torch.float32, (logits.shape[-1],))
         if logits.dim() != 2 or not 1 <= top <= logits.shape[1] or score not in ("sigmoid", "softmax"):
             raise KernelError(f"route_top: logits {tuple(logits.shape)}, top={top}, score={score!r}")
         tokens, experts = logits.shape
         choice = torch.empty((tokens, top), dtype=torch.int32, device=self.device)
         weight = torch.empty((tokens, top), dtype=torch.float32, device=self.device)
         self._launched(self._core.velox_route_top(_ptr(logits), _ptr(choice), _ptr(weight), tokens, experts, int(top), int(score == "softmax"),
-                                                  int(bool(renormalize)), self._stream()), "route_top")
+                                                  int(bool(renormalize)), _ptr(correction), self._stream()), "route_top")
         return choice, weight
 
     def routed_plan_elems(self, max_num_tokens: int, top: int, experts: int) -> int:
         """int32 elements of the plan of a step of at most ``max_num_tokens`` tokens."""
         return int(self._core.velox_routed_plan_elems(int(max_num_tokens) * int(top), int(experts)))
 
-    def routed_experts(self, x, choice, weight, gate_up_weight, down_weight, num_experts: int, scale_input: bool, shared, out_dtype, workspace=None):
+    def routed_experts(self, x, choice, weight, gate_up_weight, down_weight, num_experts: int, scale_input: bool, shared, out_dtype, workspace=None,
+                       unit: Tuple[float, float, float] = (1.0, float("inf"), 0.0), identity_experts: int = 0):
         """``sum_k unit_{choice[t, k]}(weight[t, k] x[t])`` (or the weight on the unit's output), plus ``shared``: the pairs
         are sorted by expert on the device, two grouped products run every expert on its rows, and each token's results
         are added in the order of its choices.  ``gate_up_weight`` [E * 2F, H] (per expert gate rows, then up rows),
-        ``down_weight`` [E * H, F]."""
+        ``down_weight`` [E * H, F].  ``unit = (alpha, limit, shift)``: the middle of a unit is ``g sigmoid(alpha g) (u +
+        shift)`` with ``g = min(gate, limit)``, ``u = clamp(up, -limit, limit)``.  ``identity_experts``: choices from
+        ``num_experts`` on are experts without tensors whose result is ``weight[t, k] x[t]``; the plan leaves them out and
+        the last kernel adds them in their turn."""
+        alpha, limit, shift = (float(v) for v in unit)
+        if not limit > 0 or identity_experts < 0:
+            raise KernelError(f"routed_experts: unit={unit}, identity_experts={identity_experts}")
         tokens, hidden = x.shape
         top = choice.shape[1]
         pairs = tokens * top
@@ -866,18 +970,18 @@ class HipOps:
             # bfloat16 rows of whole 16-byte pieces: sorted copies of the rows, then both products on the matrix cores
             self._launched(self._core.velox_routed_products_bf16(_P(0) if copied_by_plan else _ptr(x), _ptr(gate_up_weight), _ptr(down_weight), _ptr(ordered), _ptr(act), _ptr(y), _ptr(plan),
                                                                  _ptr(weight), pairs, num_experts, top, inter, hidden, int(bool(scale_input)), tile_rows,
-                                                                 self._stream()), "routed_products")
-            return self._routed_combine(y, plan, shared, tokens, top, num_experts, hidden, out_dtype)
+                                                                 alpha, limit, shift, self._stream()), "routed_products")
+            return self._routed_combine(y, plan, shared, tokens, top, num_experts, hidden, out_dtype, x if identity_experts else None, weight)
         self._launched(self._core.velox_grouped_glu(_ptr(x), _ptr(gate_up_weight), _ptr(act), _ptr(plan), _ptr(weight), pairs, num_experts, top, inter, hidden,
-                                                    int(bool(scale_input)), _code(x.dtype), self._stream()), "grouped_glu")
+                                                    int(bool(scale_input)), _code(x.dtype), alpha, limit, shift, self._stream()), "grouped_glu")
         self._launched(self._core.velox_grouped_down(_ptr(act), _ptr(down_weight), _ptr(y), _ptr(plan), _ptr(weight), pairs, num_experts, top, hidden, inter,
                                                      int(not scale_input), _code(x.dtype), self._stream()), "grouped_down")
-        return self._routed_combine(y, plan, shared, tokens, top, num_experts, hidden, out_dtype)
+        return self._routed_combine(y, plan, shared, tokens, top, num_experts, hidden, out_dtype, x if identity_experts else None, weight)
 
-    def _routed_combine(self, y, plan, shared, tokens, top, num_experts, hidden, out_dtype):
+    def _routed_combine(self, y, plan, shared, tokens, top, num_experts, hidden, out_dtype, identity_input=None, weight=None):
         out = torch.empty((tokens, hidden), dtype=out_dtype, device=self.device)
         self._launched(self._core.velox_routed_combine(_ptr(y), _ptr(plan), _ptr(shared), _ptr(out), tokens, top, num_experts, hidden, _code(out_dtype),
-                                                       self._stream()), "routed_combine")
+                                                       _ptr(identity_input), _ptr(weight), self._stream()), "routed_combine")
         return out
 
     # -- attention ------------------------------------------------------------------------------
@@ -927,12 +1031,14 @@ class HipOps:
 
     def paged_attention(self, qkv, num_heads, num_kv_heads, head_dim, k_cache, v_cache, block_size, block_tables, cu_q, kv_lens,
                         max_q_len, max_kv_len, scale, window, all_decode, workspace, splits: Optional[int] = None, decode_prefix: int = 0,
-                        portions_max_kv_len: Optional[int] = None):
+                        portions_max_kv_len: Optional[int] = None, distance_bias: Optional[torch.Tensor] = None):
         """Attention of every token of the step over its sequence's keys in the cache.  ``decode_prefix``: how many of the
         first sequences bring exactly one token (the engine puts decoded tokens before portions of prompts).  In a mixed
         step those run through the streaming kernel with their keys split over workgroups, the others through the
         general kernel: a single token behind many keys would otherwise be one workgroup's long walk that the
-        whole step waits for.  ``portions_max_kv_len``: the most keys any sequence behind that prefix holds (default: ``max_kv_len``)."""
+        whole step waits for.  ``portions_max_kv_len``: the most keys any sequence behind that prefix holds (default: ``max_kv_len``).
+        ``distance_bias``: float32 ``[num_heads, L]``, added to the scaled scores: a key ``n`` positions behind the query reads
+        column ``min(n, L - 1)`` of its query head's row (the kernels' build for it is loaded by ``attention_library(d, True)``)."""
         tokens = qkv.shape[0]
         width = qkv.shape[1] if qkv.dim() == 2 else -1  # rows may carry keys and values after the queries
         if width not in (num_heads * head_dim, (num_heads + 2 * num_kv_heads) * head_dim):
@@ -960,6 +1066,14 @@ class HipOps:
         if not 0 <= decode_prefix <= num_seqs or num_seqs > tokens:
             raise KernelError(f"decode_prefix={decode_prefix} does not fit {num_seqs} sequences with {tokens} tokens")
         out = torch.empty((tokens, num_heads * head_dim), dtype=qkv.dtype, device=self.device)
+        bias_len = 0
+        if distance_bias is not None:
+            self._check("distance_bias", distance_bias, torch.float32)
+            if distance_bias.dim() != 2 or distance_bias.shape[0] != num_heads or distance_bias.shape[1] < 1:
+                raise KernelError(f"paged_attention: the bias by distance is [{num_heads}, L], got {tuple(distance_bias.shape)}")
+            if head_dim > self.MAX_TILED_HEAD_DIM:
+                raise KernelError(f"paged_attention: a bias by distance needs the tiled kernels (head_dim up to {self.MAX_TILED_HEAD_DIM})")
+            bias_len = int(distance_bias.shape[1])
         if head_dim > self.MAX_TILED_HEAD_DIM:
             # beyond the tiled kernels: one workgroup per token and head, plain float32 arithmetic
             if head_dim > 1024:
@@ -969,7 +1083,7 @@ class HipOps:
                                                       block_size.bit_length() - 1, float(scale), int(window or 0), _code(qkv.dtype), self._stream())
             self._launched(status, "plain_attention")
             return out
-        lib = self.attention_library(head_dim)
+        lib = self.attention_library(head_dim, distance_bias is not None)
         group = num_heads // num_kv_heads
 
         def launch(first_seq: int, count: int, first_token: int, num_tokens: int, longest: int, decode_only: bool, splits: Optional[int]) -> None:
@@ -996,7 +1110,7 @@ class HipOps:
                 _ptr(cu_q[first_seq:]), _ptr(kv_lens[first_seq:]), _ptr(rows_out), _ptr(part_o), _ptr(part_lse), count,
                 num_tokens if decode_only else tokens, longest, int(max_kv_len), num_heads, num_kv_heads,
                 block_size.bit_length() - 1, float(scale), int(window or 0), splits, 0 if decode_only else first_token, _code(qkv.dtype),
-                self._stream())
+                _ptr(distance_bias), bias_len, self._stream())
             self._launched(status, "paged_attention")
 
         if not all_decode and splits is None and 0 < decode_prefix < num_seqs and group <= 16:
