@@ -16,7 +16,8 @@ over the steps in which all of them decode, ``..._frac``: that step's share of t
 ``e2e_b<B>_p512_g256``: generated tokens / wall time with the prompts' time included, which is how
 the reference's ``benchmark.py:204`` counts).
 
-``--design tiverax`` measures something else and leaves the above untouched: prefill and decode throughput of the Tiverax
+``--design dipisun`` does for the Dipisun design what ``--design tiverax`` does for Tiverax, beside Tiverax with the same experts and
+the dense decoder with the same heads.  ``--design tiverax`` measures something else and leaves the above untouched: prefill and decode throughput of the Tiverax
 design (attention over a cached latent, routed experts) at layer sizes of real models, beside the Qwen2 dense decoder
 with the same width, depth, heads and dense feed-forward size, as one JSON line of its own.
 """
@@ -256,16 +257,53 @@ def qwen2_like(size: dict) -> dict:
                 head_dim=size["dim"] + size["rot_dim"], intermediate_size=size["ff"], vocab_size=DESIGN_VOCAB)
 
 
+# Layer sizes for --design dipisun: eight layers, the first of every three with the bias by distance and the temperature,
+# the others without positions, every layer blending its values and every feed-forward a mixture of experts with two
+# identity experts.  Beside it: Tiverax with the same experts in every layer (its own attention, no shared expert), and
+# the dense decoder with the same heads, whose feed-forward is as wide as the experts one token uses.
+DIPISUN_SIZES = {
+    "2k": dict(width=2048, heads=16, kv_heads=4, dim=128, vdim=128, buckets=32, far=2048, experts=16, identity=2, top=2, expert_ff=1408),
+    "4k": dict(width=4096, heads=32, kv_heads=8, dim=128, vdim=128, buckets=32, far=2048, experts=32, identity=2, top=4, expert_ff=1408),
+}
+
+
+def dipisun_config(size: dict) -> dict:
+    base = {"heads": size["heads"], "kv_heads": size["kv_heads"], "dim": size["dim"], "vdim": size["vdim"], "scale": size["dim"] ** -0.5, "v_mix": True}
+    biased = dict(base, bias_max=size["far"], bias_buckets=size["buckets"], q_temp={"coef": 0.1, "every": 1024})
+    mlp = {"kind": "moe", "router": {"experts": size["experts"], "identity": size["identity"], "top": size["top"]}, "expert": {"ff": size["expert_ff"], "limit": 7.0}}
+    layers = [{"type": "attention" if index % 3 == 0 else "attention_2", "mixer": dict(biased if index % 3 == 0 else base), "mlp": mlp} for index in range(DESIGN_LAYERS)]
+    return {"architecture": "Dipisun", "vocab": DESIGN_VOCAB, "width": size["width"], "norm": {"eps": 1e-5}, "residual_mult": 0.5, "layers": layers}
+
+
+def tiverax_all_routed(size: dict) -> dict:
+    """Tiverax at the width of ``size`` with the same experts per layer and per token (no shared expert, no dense layers)."""
+    config = tiverax_config(dict(TIVERAX_SIZES["2k" if size["width"] == 2048 else "4k"], experts=size["experts"], top=size["top"], expert_ff=size["expert_ff"]))
+    routed = {"kind": "moe", "router": {"experts": size["experts"], "top": size["top"]}, "expert": {"ff": size["expert_ff"]}}
+    for entry in config["layers"]:
+        entry["mlp"] = routed
+    return config
+
+
+def designs_at(design: str, name: str):
+    if design == "tiverax":
+        size = TIVERAX_SIZES[name]
+        return (("tiverax", tiverax_config(size)), ("qwen2", qwen2_like(size)))
+    size = DIPISUN_SIZES[name]
+    dense = dict(width=size["width"], heads=size["heads"], kv_heads=size["kv_heads"], dim=size["dim"], rot_dim=0, ff=size["top"] * size["expert_ff"])
+    return (("dipisun", dipisun_config(size)), ("tiverax", tiverax_all_routed(size)), ("qwen2", qwen2_like(dense)))
+
+
 def design_points(args) -> dict:
-    """Prefill of one prompt and a decode step at batch 8, for both designs at every size, one engine after the other."""
+    """Prefill of one prompt and a decode step at batch 8, for the design and its neighbours at every size, one engine after the other."""
     import gc
 
     import torch
 
     out = {}
     for name in args.sizes.split(","):
-        size = TIVERAX_SIZES[name]
-        for label, config in (("tiverax", tiverax_config(size)), ("qwen2", qwen2_like(size))):
+        for label, config in designs_at(args.design, name):
+            if args.only and label not in args.only.split(","):
+                continue
             engine = make_engine(config, args.dtype, args.batch, args.context, args.prefill_tokens, not args.no_graphs)
             step_s, _ = time_decode(engine, DESIGN_VOCAB, args.batch, args.context, args.steps, args.warmup)
             one_s, _ = time_decode(engine, DESIGN_VOCAB, 1, args.context, max(8, args.steps // 2), args.warmup)
@@ -298,8 +336,9 @@ def main() -> int:
     parser.add_argument("--shape", default="7b", choices=sorted(SHAPES), help="layer sizes: the headline is 7b; 1.5b and 32b are the reference's other two")
     parser.add_argument("--far", action="store_true",
                         help="further sizes under `points`: decode at batch 1 and 8 behind 32,256 tokens, a prefill of 8,192 tokens, and a decode step of a true float32 run (batch 8)")
-    parser.add_argument("--design", default=None, choices=["tiverax"],
-                        help="instead of the headline: prefill and decode of this design at real layer sizes beside the Qwen2 dense decoder of equal size")
+    parser.add_argument("--design", default=None, choices=["tiverax", "dipisun"],
+                        help="instead of the headline: prefill and decode of this design at real layer sizes beside the framework's closest models of equal size")
+    parser.add_argument("--only", default="", help="with --design: which of the models that are measured side by side (names with commas between them; default: all)")
     parser.add_argument("--sizes", default="2k,4k", help="with --design: which of the sizes (2k, 4k = the models' widths)")
     args = parser.parse_args()
     if args.design is not None:
@@ -310,12 +349,14 @@ def main() -> int:
             args.context = 2048  # (the design's default context, unless the caller names another)
         points = design_points(args)
         first = args.sizes.split(",")[0]
+        head = points.get(f"{args.design}_{first}") or next(iter(points.values()))
+        sizes = TIVERAX_SIZES if args.design == "tiverax" else DIPISUN_SIZES
         print(json.dumps({
-            "metric": "decode_tokens_per_second", "value": points[f"tiverax_{first}"]["decode_tok_s"], "unit": "tok/s", "n_gpus": 1, "steps": args.steps,
-            "warmup": args.warmup, "ms_per_step": points[f"tiverax_{first}"]["decode_ms"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "metric": "decode_tokens_per_second", "value": head["decode_tok_s"], "unit": "tok/s", "n_gpus": 1, "steps": args.steps,
+            "warmup": args.warmup, "ms_per_step": head["decode_ms"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
             "dtype": args.dtype, "data": "synthetic: random weights N(0,0.02), uniform random token ids",
-            "config": {"model": f"Tiverax design, size {first}", "layers": DESIGN_LAYERS, "global_batch": args.batch, "seq_len": args.context,
-                       "prefill_tokens": args.prefill_tokens, "sizes": {name: TIVERAX_SIZES[name] for name in args.sizes.split(",")}, "parallelism": "single-gpu"},
+            "config": {"model": f"{args.design.capitalize()} design, size {first}", "layers": DESIGN_LAYERS, "global_batch": args.batch, "seq_len": args.context,
+                       "prefill_tokens": args.prefill_tokens, "sizes": {name: sizes[name] for name in args.sizes.split(",")}, "parallelism": "single-gpu"},
             "points": points}))
         return 0
     if args.gpus != 1:

@@ -385,21 +385,22 @@ extern "C" int velox_routed_products_bf16(const void* x, const void* gate_up, co
   glu.unit = GluUnit{alpha, limit, shift};
   grouped_mfma_launch<GM_GLU, bf16_t>(glu, pairs, tile_rows, max_tiles, 1, stream);
   GroupedArgs last = routed_args(act, down, y, plan, pairs, experts, hidden, inter, hidden);
-  last.row_scale = pair_weight;
-  if (scale_input) grouped_mfma_launch<GM_PLAIN, float>(last, pairs, tile_rows, max_tiles, 1, stream);
-  else grouped_mfma_launch<GM_ROW_SCALE, float>(last, pairs, tile_rows, max_tiles, 1, stream);
+  // (a weight on the experts' OUTPUT is applied where the results are added up, routed_combine with scale_rows: the product
+  // itself is the same kernel either way)
+  grouped_mfma_launch<GM_PLAIN, float>(last, pairs, tile_rows, max_tiles, 1, stream);
   VELOX_RETURN_LAUNCH_STATUS();
 }
 
 // ---------------------------------------------------------------------------------------------
 // out[t, :] = (sum_k y[place[t * top + k], :]) + shared[t, :], the choices added in order, one rounding at the store.
 // With `x`: a choice that the plan has not placed (an identity expert, whose index lies behind the real ones) adds
-// pair_weight[t * top + k] * x[t, :] in its turn.
+// pair_weight[t * top + k] * x[t, :] in its turn.  With `scale_rows` every row of y is multiplied with its pair's weight here
+// (the products then left it out).
 // ---------------------------------------------------------------------------------------------
 template <typename T>
 __global__ void __launch_bounds__(256) routed_combine_kernel(const float* __restrict__ y, const int* __restrict__ place, const T* __restrict__ shared,
                                                              T* __restrict__ out, int top, int hidden, const T* __restrict__ x,
-                                                             const float* __restrict__ pair_weight) {
+                                                             const float* __restrict__ pair_weight, int scale_rows) {
   __shared__ int rows[64];  // the token's rows of y, looked up once (up to 64 choices; more are looked up as they are added)
   const int t = blockIdx.x;
   const int* mine = place + (size_t)t * top;
@@ -412,7 +413,7 @@ __global__ void __launch_bounds__(256) routed_combine_kernel(const float* __rest
     float v = 0.f;
     for (int k = 0; k < top; ++k) {
       const int row = mine[k];
-      if (row >= 0) v += y[(size_t)row * hidden + i];
+      if (row >= 0) v += scale_rows ? pair_weight[(size_t)t * top + k] * y[(size_t)row * hidden + i] : y[(size_t)row * hidden + i];
       else if (x) v += pair_weight[(size_t)t * top + k] * to_f32(x[(size_t)t * hidden + i]);
     }
     if (shared) v += to_f32(shared[(size_t)t * hidden + i]);
@@ -421,12 +422,12 @@ __global__ void __launch_bounds__(256) routed_combine_kernel(const float* __rest
 }
 
 extern "C" int velox_routed_combine(const float* y, const int* plan, const void* shared, void* out, int tokens, int top, int experts, int hidden, int dtype,
-                                    const void* x, const float* pair_weight, hipStream_t stream) {
+                                    const void* x, const float* pair_weight, int scale_rows, hipStream_t stream) {
   if (tokens <= 0) return 0;
   const int* place = plan + 1 + (experts + 1) + (size_t)tokens * top;
   if (dtype == VELOX_BF16)
-    routed_combine_kernel<bf16_t><<<tokens, 256, 0, stream>>>(y, place, (const bf16_t*)shared, (bf16_t*)out, top, hidden, (const bf16_t*)x, pair_weight);
+    routed_combine_kernel<bf16_t><<<tokens, 256, 0, stream>>>(y, place, (const bf16_t*)shared, (bf16_t*)out, top, hidden, (const bf16_t*)x, pair_weight, scale_rows);
   else
-    routed_combine_kernel<float><<<tokens, 256, 0, stream>>>(y, place, (const float*)shared, (float*)out, top, hidden, (const float*)x, pair_weight);
+    routed_combine_kernel<float><<<tokens, 256, 0, stream>>>(y, place, (const float*)shared, (float*)out, top, hidden, (const float*)x, pair_weight, scale_rows);
   VELOX_RETURN_LAUNCH_STATUS();
 }

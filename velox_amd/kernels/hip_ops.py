@@ -150,7 +150,7 @@ class HipOps:
         c.velox_routed_plan.argtypes = [_P, _I, _I, _P, _I, _P, _P, _P, _I, _I, _I, _P]
         c.velox_grouped_glu.argtypes = [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _F, _F, _P]
         c.velox_grouped_down.argtypes = [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P]
-        c.velox_routed_combine.argtypes = [_P, _P, _P, _P, _I, _I, _I, _I, _I, _P, _P, _P]
+        c.velox_routed_combine.argtypes = [_P, _P, _P, _P, _I, _I, _I, _I, _I, _P, _P, _I, _P]
         c.velox_routed_products_bf16.argtypes = [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _F, _F, _P]
         c.velox_add_sinusoid.argtypes = [_P, _P, _P, _I, _I, _P]
         c.velox_add_cast.argtypes = [_P, _P, _I, _P, ctypes.c_longlong, _P]
@@ -971,17 +971,19 @@ class HipOps:
             self._launched(self._core.velox_routed_products_bf16(_P(0) if copied_by_plan else _ptr(x), _ptr(gate_up_weight), _ptr(down_weight), _ptr(ordered), _ptr(act), _ptr(y), _ptr(plan),
                                                                  _ptr(weight), pairs, num_experts, top, inter, hidden, int(bool(scale_input)), tile_rows,
                                                                  alpha, limit, shift, self._stream()), "routed_products")
-            return self._routed_combine(y, plan, shared, tokens, top, num_experts, hidden, out_dtype, x if identity_experts else None, weight)
+            # (a weight on the output is applied by the last kernel: the second product is the same kernel either way)
+            return self._routed_combine(y, plan, shared, tokens, top, num_experts, hidden, out_dtype, x if identity_experts else None, weight,
+                                        scale_rows=not scale_input)
         self._launched(self._core.velox_grouped_glu(_ptr(x), _ptr(gate_up_weight), _ptr(act), _ptr(plan), _ptr(weight), pairs, num_experts, top, inter, hidden,
                                                     int(bool(scale_input)), _code(x.dtype), alpha, limit, shift, self._stream()), "grouped_glu")
         self._launched(self._core.velox_grouped_down(_ptr(act), _ptr(down_weight), _ptr(y), _ptr(plan), _ptr(weight), pairs, num_experts, top, hidden, inter,
                                                      int(not scale_input), _code(x.dtype), self._stream()), "grouped_down")
         return self._routed_combine(y, plan, shared, tokens, top, num_experts, hidden, out_dtype, x if identity_experts else None, weight)
 
-    def _routed_combine(self, y, plan, shared, tokens, top, num_experts, hidden, out_dtype, identity_input=None, weight=None):
+    def _routed_combine(self, y, plan, shared, tokens, top, num_experts, hidden, out_dtype, identity_input=None, weight=None, scale_rows=False):
         out = torch.empty((tokens, hidden), dtype=out_dtype, device=self.device)
         self._launched(self._core.velox_routed_combine(_ptr(y), _ptr(plan), _ptr(shared), _ptr(out), tokens, top, num_experts, hidden, _code(out_dtype),
-                                                       _ptr(identity_input), _ptr(weight), self._stream()), "routed_combine")
+                                                       _ptr(identity_input), _ptr(weight), int(bool(scale_rows)), self._stream()), "routed_combine")
         return out
 
     # -- attention ------------------------------------------------------------------------------
