@@ -21,6 +21,7 @@ from velox_amd.cache import CacheManager
 from velox_amd.engine.batch import BatchBuilder, StepEntry, Workspace
 from velox_amd.engine.replay import Replayer
 from velox_amd.parts import make_part
+from velox_amd.parts.base import OutputNormSink, ResidualCopy
 from velox_amd.parts.normed_attention import bias_by_distance
 
 pytestmark = pytest.mark.gpu
@@ -134,6 +135,17 @@ def test_clamped_units_and_identity_experts_against_the_plain_loop(ops, dtype, t
     got = ops.routed_experts(x, choice, weight, gate_up, down, experts, False, None, dt, None, unit=unit, identity_experts=identity)
     want = ref.routed_experts(x, choice, weight, gate_up, down, experts, False, None, dt, None, unit=unit, identity_experts=identity)
     close(got, want, dtype, scale=0.5)
+    # the same with the last kernel norming the sum and adding it to a residual
+    norm_weight = (1 + 0.1 * torch.randn(hidden)).cuda()
+    mine, theirs = torch.randn(tokens, hidden).cuda(), None
+    theirs = mine.clone()
+    fused = ops.routed_experts(x, choice, weight, gate_up, down, experts, False, None, dt, None, unit=unit, identity_experts=identity,
+                               output_norm=OutputNormSink(mine, norm_weight, 1e-5, 0.7))
+    plain = ref.routed_experts(x, choice, weight, gate_up, down, experts, False, None, dt, None, unit=unit, identity_experts=identity,
+                               output_norm=OutputNormSink(theirs, norm_weight, 1e-5, 0.7))
+    assert isinstance(fused, ResidualCopy) and fused.copy.dtype == dt and (fused.copy is mine) == (dtype == "float32")
+    close(mine, theirs, dtype, scale=0.5)
+    close(fused.copy, plain.copy, dtype, scale=0.5)
     unclamped = ref.routed_experts(x, choice, weight, gate_up, down, experts, False, None, dt, None, unit=(1.702, 1e9, 1.0), identity_experts=identity)
     assert tokens < 9 or float((unclamped.float() - want.float()).abs().max()) > 0.05  # the clamps are reached
 
@@ -253,9 +265,11 @@ def test_all_ways_of_cutting_on_the_gpu(tmp_path, name, dtype):
             if dtype == "float32":
                 torch.testing.assert_close(got, want, msg=lambda m: f"{name} {label} {rid}: {m}", rtol=2e-4, atol=3e-5 * size)
             else:
-                # bfloat16: rounding may send a token to another expert where two scores are close; such rows are few
+                # bfloat16: rounding may send a token to another expert where two scores are close (the tests' routers and
+                # corrections are sharp, so that float32 shows every fault; bfloat16 then flips some choices): most rows are
+                # close, the typical row is very close
                 err = (got - want).abs().amax(-1) / want.abs().amax(-1).clamp(min=1.0)
-                assert float((err < 0.08).float().mean()) >= 0.9, f"{name} {label} {rid}: {err}"
+                assert float((err < 0.08).float().mean()) >= 0.8 and (len(err) < 8 or float(err.median()) < 0.04), f"{name} {label} {rid}: {err}"
         if label in ("mixed", "recompute"):
             assert sum((len(t) + page - 1) // page for t in requests.values()) > replayer.cache.num_total_pages
     if dtype == "float32":
@@ -282,7 +296,7 @@ def test_long_decoding_and_a_batch_against_each_request_alone(tmp_path, dtype):
         torch.testing.assert_close(got, want[[0] + list(range(4, 205))], rtol=2e-4, atol=3e-5 * float(want.abs().max()))
     else:
         err = (got - want[[0] + list(range(4, 205))]).abs().amax(-1) / want.abs().amax()
-        assert float((err < 0.08).float().mean()) >= 0.9
+        assert float((err < 0.08).float().mean()) >= 0.8 and float(err.median()) < 0.04
     texts = prompts(config["vocab"], [70, 9, 33, 120], seed=13)
     alone = {}
     for rid, text in texts.items():

@@ -270,7 +270,7 @@ class TorchOps:
         return choice.to(torch.int32), weight
 
     def routed_experts(self, x, choice, weight, gate_up_weight, down_weight, num_experts, scale_input, shared, out_dtype, workspace=None,
-                       unit=(1.0, float("inf"), 0.0), identity_experts=0):
+                       unit=(1.0, float("inf"), 0.0), identity_experts=0, output_norm=None):
         alpha, limit, shift = unit
         t, h = x.shape
         f = gate_up_weight.shape[0] // (2 * num_experts)
@@ -294,6 +294,10 @@ class TorchOps:
                 out[rows] += y if scale_input else y * w
         if shared is not None:
             out = out + shared.float()
+        if output_norm is not None:  # the sum goes to the norm as it is, in float32
+            from velox_amd.parts.base import ResidualCopy
+
+            return ResidualCopy(self.norm_add(output_norm.residual, out, output_norm.weight, output_norm.eps, output_norm.mult, out_dtype))
         return out.to(out_dtype)
 
     # -- attention over the paged cache -------------------------------------------------

@@ -421,6 +421,71 @@ __global__ void __launch_bounds__(256) routed_combine_kernel(const float* __rest
   }
 }
 
+// The same sum, handed straight to a norm on the experts' output: residual[t, :] += mult * v * rsqrt(mean(v^2) + eps) * w, with v the
+// sum above in float32 (never rounded to T), and `copy` (nullable) the updated residual in T.  One workgroup per token holds
+// the row in registers: hidden <= 16 * blockDim.x.
+template <typename T>
+__global__ void routed_combine_norm_kernel(const float* __restrict__ y, const int* __restrict__ place, const T* __restrict__ shared, int top, int hidden,
+                                           const T* __restrict__ x, const float* __restrict__ pair_weight, int scale_rows, float* __restrict__ residual,
+                                           const float* __restrict__ norm_weight, float eps, float mult, T* __restrict__ copy) {
+  __shared__ int rows[64];
+  __shared__ float scratch[16];
+  const int t = blockIdx.x;
+  const int* mine = place + (size_t)t * top;
+  if (top <= 64) {
+    if (threadIdx.x < top) rows[threadIdx.x] = mine[threadIdx.x];
+    __syncthreads();
+    mine = rows;
+  }
+  float held[16];
+  float sumsq = 0.f;
+#pragma unroll
+  for (int c = 0; c < 16; ++c) {
+    const int i = threadIdx.x + c * blockDim.x;
+    float v = 0.f;
+    if (i < hidden) {
+      for (int k = 0; k < top; ++k) {
+        const int row = mine[k];
+        if (row >= 0) v += scale_rows ? pair_weight[(size_t)t * top + k] * y[(size_t)row * hidden + i] : y[(size_t)row * hidden + i];
+        else if (x) v += pair_weight[(size_t)t * top + k] * to_f32(x[(size_t)t * hidden + i]);
+      }
+      if (shared) v += to_f32(shared[(size_t)t * hidden + i]);
+    }
+    held[c] = v;
+    sumsq += v * v;
+  }
+  const float total = block_sum(sumsq, scratch);
+  const float inv = 1.f / sqrtf(total / (float)hidden + eps);
+#pragma unroll
+  for (int c = 0; c < 16; ++c) {
+    const int i = threadIdx.x + c * blockDim.x;
+    if (i < hidden) {
+      const float r = residual[(size_t)t * hidden + i] + mult * (held[c] * inv * norm_weight[i]);
+      residual[(size_t)t * hidden + i] = r;
+      if (copy) copy[(size_t)t * hidden + i] = from_f32<T>(r);
+    }
+  }
+}
+
+// copy: nullptr in a float32 run (the residual is its own copy).  Returns -1 when the row does not fit the registers
+// (hidden > 16,384): the caller then runs the two kernels one after the other.
+extern "C" int velox_routed_combine_norm(const float* y, const int* plan, const void* shared, int tokens, int top, int experts, int hidden, int dtype,
+                                         const void* x, const float* pair_weight, int scale_rows, float* residual, const float* norm_weight, float eps,
+                                         float mult, void* copy, hipStream_t stream) {
+  if (tokens <= 0) return 0;
+  if (hidden > 16 * 1024) return -1;
+  const int* place = plan + 1 + (experts + 1) + (size_t)tokens * top;
+  int threads = tokens <= 64 ? 512 : 256;  // (few rows: more threads each with less to do)
+  while (16 * threads < hidden) threads *= 2;
+  if (dtype == VELOX_BF16)
+    routed_combine_norm_kernel<bf16_t><<<tokens, threads, 0, stream>>>(y, place, (const bf16_t*)shared, top, hidden, (const bf16_t*)x, pair_weight, scale_rows,
+                                                                       residual, norm_weight, eps, mult, (bf16_t*)copy);
+  else
+    routed_combine_norm_kernel<float><<<tokens, threads, 0, stream>>>(y, place, (const float*)shared, top, hidden, (const float*)x, pair_weight, scale_rows,
+                                                                      residual, norm_weight, eps, mult, (float*)copy);
+  VELOX_RETURN_LAUNCH_STATUS();
+}
+
 extern "C" int velox_routed_combine(const float* y, const int* plan, const void* shared, void* out, int tokens, int top, int experts, int hidden, int dtype,
                                     const void* x, const float* pair_weight, int scale_rows, hipStream_t stream) {
   if (tokens <= 0) return 0;

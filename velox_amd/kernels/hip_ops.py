@@ -20,7 +20,7 @@ from typing import Tuple, Dict, Optional
 
 import torch
 
-from ..parts.base import DeferredNorm, ResidualSink, SumOf
+from ..parts.base import DeferredNorm, ResidualCopy, ResidualSink, SumOf
 from . import build
 
 logger = logging.getLogger(__name__)
@@ -152,6 +152,8 @@ class HipOps:
         c.velox_grouped_down.argtypes = [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P]
         c.velox_routed_combine.argtypes = [_P, _P, _P, _P, _I, _I, _I, _I, _I, _P, _P, _I, _P]
         c.velox_routed_products_bf16.argtypes = [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _F, _F, _P]
+        c.velox_routed_combine_norm.argtypes = [_P, _P, _P, _I, _I, _I, _I, _I, _P, _P, _I, _P, _P, _F, _F, _P, _P]
+        c.velox_routed_combine_norm.restype = _I
         c.velox_add_sinusoid.argtypes = [_P, _P, _P, _I, _I, _P]
         c.velox_add_cast.argtypes = [_P, _P, _I, _P, ctypes.c_longlong, _P]
         c.velox_norm_add.argtypes = [_P, _P, _I, _P, _P, _I, _I, _F, _F, _I, ctypes.c_longlong, _P]
@@ -926,14 +928,15 @@ class HipOps:
         return int(self._core.velox_routed_plan_elems(int(max_num_tokens) * int(top), int(experts)))
 
     def routed_experts(self, x, choice, weight, gate_up_weight, down_weight, num_experts: int, scale_input: bool, shared, out_dtype, workspace=None,
-                       unit: Tuple[float, float, float] = (1.0, float("inf"), 0.0), identity_experts: int = 0):
+                       unit: Tuple[float, float, float] = (1.0, float("inf"), 0.0), identity_experts: int = 0, output_norm=None):
         """``sum_k unit_{choice[t, k]}(weight[t, k] x[t])`` (or the weight on the unit's output), plus ``shared``: the pairs
         are sorted by expert on the device, two grouped products run every expert on its rows, and each token's results
         are added in the order of its choices.  ``gate_up_weight`` [E * 2F, H] (per expert gate rows, then up rows),
         ``down_weight`` [E * H, F].  ``unit = (alpha, limit, shift)``: the middle of a unit is ``g sigmoid(alpha g) (u +
         shift)`` with ``g = min(gate, limit)``, ``u = clamp(up, -limit, limit)``.  ``identity_experts``: choices from
         ``num_experts`` on are experts without tensors whose result is ``weight[t, k] x[t]``; the plan leaves them out and
-        the last kernel adds them in their turn."""
+        the last kernel adds them in their turn.  ``output_norm`` (an ``OutputNormSink``): the last kernel norms the sum in
+        float32 and adds it to the sink's residual; what comes back is then a ``ResidualCopy`` of the updated residual."""
         alpha, limit, shift = (float(v) for v in unit)
         if not limit > 0 or identity_experts < 0:
             raise KernelError(f"routed_experts: unit={unit}, identity_experts={identity_experts}")
@@ -973,14 +976,30 @@ class HipOps:
                                                                  alpha, limit, shift, self._stream()), "routed_products")
             # (a weight on the output is applied by the last kernel: the second product is the same kernel either way)
             return self._routed_combine(y, plan, shared, tokens, top, num_experts, hidden, out_dtype, x if identity_experts else None, weight,
-                                        scale_rows=not scale_input)
+                                        scale_rows=not scale_input, output_norm=output_norm)
         self._launched(self._core.velox_grouped_glu(_ptr(x), _ptr(gate_up_weight), _ptr(act), _ptr(plan), _ptr(weight), pairs, num_experts, top, inter, hidden,
                                                     int(bool(scale_input)), _code(x.dtype), alpha, limit, shift, self._stream()), "grouped_glu")
         self._launched(self._core.velox_grouped_down(_ptr(act), _ptr(down_weight), _ptr(y), _ptr(plan), _ptr(weight), pairs, num_experts, top, hidden, inter,
                                                      int(not scale_input), _code(x.dtype), self._stream()), "grouped_down")
-        return self._routed_combine(y, plan, shared, tokens, top, num_experts, hidden, out_dtype, x if identity_experts else None, weight)
+        return self._routed_combine(y, plan, shared, tokens, top, num_experts, hidden, out_dtype, x if identity_experts else None, weight,
+                                    output_norm=output_norm)
 
-    def _routed_combine(self, y, plan, shared, tokens, top, num_experts, hidden, out_dtype, identity_input=None, weight=None, scale_rows=False):
+    def _routed_combine(self, y, plan, shared, tokens, top, num_experts, hidden, out_dtype, identity_input=None, weight=None, scale_rows=False,
+                        output_norm=None):
+        if output_norm is not None:
+            self._check("residual", output_norm.residual, torch.float32, (tokens, hidden))
+            self._check("norm weight", output_norm.weight, torch.float32, (hidden,))
+            copy = torch.empty((tokens, hidden), dtype=out_dtype, device=self.device) if out_dtype != torch.float32 else None
+            status = self._core.velox_routed_combine_norm(_ptr(y), _ptr(plan), _ptr(shared), tokens, top, num_experts, hidden, _code(out_dtype),
+                                                          _ptr(identity_input), _ptr(weight), int(bool(scale_rows)), _ptr(output_norm.residual),
+                                                          _ptr(output_norm.weight), float(output_norm.eps), float(output_norm.mult), _ptr(copy), self._stream())
+            if status == 0:
+                return ResidualCopy(output_norm.residual if copy is None else copy)
+            if status != -1:
+                self._launched(status, "routed_combine_norm")
+            # (a row too long for the fused kernel's registers: the two kernels one after the other)
+            out = self._routed_combine(y, plan, shared, tokens, top, num_experts, hidden, out_dtype, identity_input, weight, scale_rows)
+            return ResidualCopy(self.norm_add(output_norm.residual, out, output_norm.weight, output_norm.eps, output_norm.mult, out_dtype))
         out = torch.empty((tokens, hidden), dtype=out_dtype, device=self.device)
         self._launched(self._core.velox_routed_combine(_ptr(y), _ptr(plan), _ptr(shared), _ptr(out), tokens, top, num_experts, hidden, _code(out_dtype),
                                                        _ptr(identity_input), _ptr(weight), int(bool(scale_rows)), self._stream()), "routed_combine")

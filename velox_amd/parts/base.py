@@ -232,6 +232,19 @@ class ResidualCopy:
     copy: torch.Tensor
 
 
+@dataclass
+class OutputNormSink:
+    """Where a sub-layer whose last kernel can norm its own output may put it: ``residual += mult * output *
+    rsqrt(mean(output^2) + eps) * weight``.  A feed-forward that sets ``accepts_output_norm = True`` takes ``output_norm=``
+    in ``forward`` and returns either its output as always, or, when it has done the norm and the add itself, a
+    ``ResidualCopy`` of the updated residual."""
+
+    residual: torch.Tensor
+    weight: torch.Tensor
+    eps: float
+    mult: float
+
+
 class Mixer(Part):
     def cache_need(self):
         """``PagedNeed``, ``StateNeed`` or None."""

@@ -18,7 +18,7 @@ from typing import Optional, Tuple
 
 import torch
 
-from .base import Block, FeedForward, Mixer, Norm, Part, ResidualCopy, ResidualSink, SumOf, register_arrangement
+from .base import Block, FeedForward, Mixer, Norm, OutputNormSink, Part, ResidualCopy, ResidualSink, SumOf, register_arrangement
 
 
 class PreNormBlock(Block):
@@ -121,7 +121,13 @@ class OutputNormBlock(Block):
         mixed = self.mixer.forward(x, ctx, cache, owns_cache)
         x = self.mixer_norm.add_normed(residual, mixed, self.residual_mult, ctx)
         if self.has_feed_forward:
-            out = self.feed_forward.forward(x, ctx)
+            form = self.ff_norm.deferred_form()  # (weight, eps) of a weighted RMS norm, which a sub-layer's last kernel may take over
+            if form is not None and getattr(self.feed_forward, "accepts_output_norm", False):
+                out = self.feed_forward.forward(x, ctx, output_norm=OutputNormSink(residual, form[0], form[1], self.residual_mult))
+            else:
+                out = self.feed_forward.forward(x, ctx)
+            if isinstance(out, ResidualCopy):
+                return out
             x = self.ff_norm.add_normed(residual, out, self.residual_mult, ctx)
         return ResidualCopy(x)
 

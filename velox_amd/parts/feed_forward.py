@@ -146,7 +146,9 @@ class RoutedExperts(FeedForward):
             return {}
         return {"routed_plan": sizes(limits.max_num_tokens, self.top, self.num_experts)}
 
-    def forward(self, x, ctx, sink=None):
+    accepts_output_norm = True  # its last kernel can norm the sum of the experts' results and add it to the residual
+
+    def forward(self, x, ctx, sink=None, output_norm=None):
         ops = ctx.ops
         x = ops.materialize(x)
         logits = ops.linear(x, self.router_weight, None, torch.float32)
@@ -155,6 +157,9 @@ class RoutedExperts(FeedForward):
         else:
             choice, weight = ops.route_top(logits, self.top, self.score, self.renormalize)
         shared = self.shared.forward(x, ctx, partials_ok=False) if self.shared is not None else None
+        if output_norm is not None:
+            return ops.routed_experts(x, choice, weight, self.gate_up_weight, self.down_weight, self.num_experts, self.scale_input, shared,
+                                      ctx.dtype, ctx.workspace, unit=self.unit, identity_experts=self.identity_experts, output_norm=output_norm)
         if self.unit == SILU_UNIT and not self.identity_experts:
             return ops.routed_experts(x, choice, weight, self.gate_up_weight, self.down_weight, self.num_experts, self.scale_input, shared,
                                       ctx.dtype, ctx.workspace)

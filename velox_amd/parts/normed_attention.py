@@ -103,8 +103,8 @@ class NormedAttentionMixer(Mixer):
         if self.q_temp is not None and self.q_temp[1] < 1:
             raise ValueError("q_temp: 'every' must be at least 1")
         self.distance_bias = (int(distance_bias[0]), float(distance_bias[1])) if distance_bias is not None else None
-        if self.distance_bias is not None and (self.distance_bias[0] < 2 or not self.distance_bias[1] > self.distance_bias[0] // 2):
-            raise ValueError("distance_bias: at least two buckets, and 'far' beyond the last distance that has a bucket of its own")
+        if self.distance_bias is not None and (self.distance_bias[0] < 1 or not self.distance_bias[1] > 0):
+            raise ValueError("distance_bias: at least one bucket and a positive 'far'")
         self.value_mix = value_mix
         self.value_mix_key = value_mix_key
         self.has_mix_weight = (value_mix is not None) if has_mix_weight is None else bool(has_mix_weight)
