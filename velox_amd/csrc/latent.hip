@@ -243,7 +243,7 @@ template <typename T>
 __global__ void __launch_bounds__(256) plain_attention_kernel(const T* __restrict__ q, int q_width, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
                                                               const int* __restrict__ block_tables, int table_width, const int* __restrict__ cu_q,
                                                               const int* __restrict__ kv_lens, T* __restrict__ out, int num_seqs, int nh, int nkv, int d,
-                                                              int page_shift, float scale, int window) {
+                                                              int page_shift, float scale, int window, const float* __restrict__ bias_table, int bias_len) {
   __shared__ float q_s[PLAIN_ATTENTION_MAX_D];
   __shared__ float p_s[256];
   __shared__ float scratch[16];
@@ -275,6 +275,8 @@ __global__ void __launch_bounds__(256) plain_attention_kernel(const T* __restric
       float dot = 0.f;
       for (int c = 0; c < d; ++c) dot = fmaf(q_s[c], to_f32(key[c]), dot);
       s = dot * scale;
+      // a bias by distance, float32 [nh, bias_len]: the key n positions behind the query reads column min(n, bias_len - 1)
+      if (bias_table) s += bias_table[(size_t)head * bias_len + min(last - j, bias_len - 1)];
     }
     const float new_max = fmaxf(running_max, block_max_256(s, scratch));  // (finite: key j0 is always seen)
     const float p = j <= last ? expf(s - new_max) : 0.f;
@@ -306,15 +308,16 @@ __global__ void __launch_bounds__(256) plain_attention_kernel(const T* __restric
 
 extern "C" int velox_plain_attention(const void* q, int q_width, const void* k_cache, const void* v_cache, const int* block_tables, int table_width,
                                      const int* cu_q, const int* kv_lens, void* out, int num_seqs, int tokens, int nh, int nkv, int d, int page_shift,
-                                     float scale, int window, int dtype, hipStream_t stream) {
+                                     float scale, int window, int dtype, const float* bias_table, int bias_len, hipStream_t stream) {
   if (tokens <= 0) return 0;
+  if (bias_table != nullptr && bias_len < 1) return -1;
   if (d < 1 || d > PLAIN_ATTENTION_MAX_D || nh < 1 || nkv < 1 || nh % nkv != 0 || nh > 65535 || num_seqs < 1 || nh * d > q_width) return -1;
   dim3 grid(tokens, nh);
   if (dtype == VELOX_BF16)
     plain_attention_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)q, q_width, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables, table_width,
-                                                             cu_q, kv_lens, (bf16_t*)out, num_seqs, nh, nkv, d, page_shift, scale, window);
+                                                             cu_q, kv_lens, (bf16_t*)out, num_seqs, nh, nkv, d, page_shift, scale, window, bias_table, bias_len);
   else
     plain_attention_kernel<float><<<grid, 256, 0, stream>>>((const float*)q, q_width, (const float*)k_cache, (const float*)v_cache, block_tables, table_width,
-                                                            cu_q, kv_lens, (float*)out, num_seqs, nh, nkv, d, page_shift, scale, window);
+                                                            cu_q, kv_lens, (float*)out, num_seqs, nh, nkv, d, page_shift, scale, window, bias_table, bias_len);
   VELOX_RETURN_LAUNCH_STATUS();
 }

@@ -142,7 +142,7 @@ class HipOps:
         c.velox_probe_grid_barrier.restype = _I
         c.velox_latent_rotate_write.argtypes = [_P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _P, _P, _P, _I, _I, _P, _F, _P, _P, _P, _I, _I, _P]
         c.velox_head_linear.argtypes = [_P, _I, _I, _I, _P, _P, _I, _I, _I, _P, _I, _I, _I, _I, _I, _I, _I, _P]
-        c.velox_plain_attention.argtypes = [_P, _I, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _P]
+        c.velox_plain_attention.argtypes = [_P, _I, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _P, _I, _P]
         c.velox_plain_attention.restype = _I
         c.velox_route_top.argtypes = [_P, _P, _P, _I, _I, _I, _I, _I, _P, _P]
         c.velox_routed_plan_elems.argtypes = [_I, _I]
@@ -1092,8 +1092,6 @@ class HipOps:
             self._check("distance_bias", distance_bias, torch.float32)
             if distance_bias.dim() != 2 or distance_bias.shape[0] != num_heads or distance_bias.shape[1] < 1:
                 raise KernelError(f"paged_attention: the bias by distance is [{num_heads}, L], got {tuple(distance_bias.shape)}")
-            if head_dim > self.MAX_TILED_HEAD_DIM:
-                raise KernelError(f"paged_attention: a bias by distance needs the tiled kernels (head_dim up to {self.MAX_TILED_HEAD_DIM})")
             bias_len = int(distance_bias.shape[1])
         if head_dim > self.MAX_TILED_HEAD_DIM:
             # beyond the tiled kernels: one workgroup per token and head, plain float32 arithmetic
@@ -1101,7 +1099,8 @@ class HipOps:
                 raise KernelError(f"paged_attention: head_dim={head_dim} is beyond every kernel (1,024 at most)")
             status = self._core.velox_plain_attention(_ptr(qkv), width, _ptr(k_cache), _ptr(v_cache), _ptr(block_tables), block_tables.shape[1], _ptr(cu_q),
                                                       _ptr(kv_lens), _ptr(out), num_seqs, tokens, num_heads, num_kv_heads, head_dim,
-                                                      block_size.bit_length() - 1, float(scale), int(window or 0), _code(qkv.dtype), self._stream())
+                                                      block_size.bit_length() - 1, float(scale), int(window or 0), _code(qkv.dtype), _ptr(distance_bias), bias_len,
+                                                      self._stream())
             self._launched(status, "plain_attention")
             return out
         lib = self.attention_library(head_dim, distance_bias is not None)
