@@ -49,6 +49,8 @@ def distance_bucket(n: int, buckets: int, far: float) -> int:
     near = buckets // 2
     if n < near:
         return n
+    if near == 0 or far <= near:  # (no logarithmic part to speak of: everything else is the last bucket)
+        return buckets - 1
     return min(buckets - 1, near + int(math.floor(math.log(n / near) / math.log(far / near) * (buckets - near))))
 
 
